@@ -96,8 +96,7 @@ __global__ void skinny_gemm3_kernel(
     // SPLIT prefetch queues (the single-queue version collapsed: 6 fused
     // stages x 12 VGPRs + temps exceeded the 128-VGPR budget and the
     // allocator reused stage registers, shrinking the pipeline to depth
-    // ~1.5 — the ISA showed `s_waitcnt vmcnt(2)`/`vmcnt(0)` at every
-    // commit). W is the HBM stream and needs the deep queue (8 stages x
+    // ~1.5 by its timing). W is the HBM stream and needs the deep queue (8 stages x
     // 4 VGPRs); x is XCD-L2-resident (192 WGs re-read the same 1 MB) so
     // a short 4-stage queue covers its latency.
     auto load_w = [&](int k0, sk3_i32x4* r) {
