@@ -1,4 +1,8 @@
-"""Gated delta-rule token mixer core (a linear recurrence with matrix state).
+"""Linear-recurrence token mixer cores with matrix state: the gated delta
+rule (below), selective state spaces (:class:`StateSpaceDuality`) and
+retention (:class:`Retention`).
+
+Gated delta rule.
 
 Per head the state is a (dim x vdim) fp32 matrix ``M`` updated once per token
 
@@ -97,3 +101,99 @@ class GatedDeltaRule(nn.Module):
             qkv_c, beta, a, self.dt_bias, self.A_log, gate, self.norm_weight,
             self.eps, states.get(key + ".mem"), step, self.num_kv_heads, self.dim,
             self.vdim, out_dtype=a.dtype, gate_act=self.gate_act)
+
+
+class StateSpaceDuality(nn.Module):
+    """Selective state-space token mixer core (the scalar-decay, multi-head
+    form that is dual to a masked linear attention).
+
+    Per head the state is an (state x vdim) fp32 matrix
+
+        S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T ,
+        y_t = S_t^T C_t + D x_t ,   dt_t = softplus(dt_proj_t + dt_bias)
+
+    with one decay, step size and skip weight ``D`` per head; ``B`` and ``C``
+    (``groups`` of them, each shared by heads/groups consecutive heads) and
+    ``x`` first pass one short causal convolution with bias and SiLU. The
+    output is multiplied by silu(z) and THEN RMS-normed in ``norm_groups``
+    equal channel groups and weighted.
+
+    The caller owns the input projection, laid out [z | x | B | C | dt], and
+    the output projection. State (``S`` and the convolution tail) lives in the
+    cache manager's :class:`RecurrentStateManager`.
+    """
+
+    def __init__(self, num_heads: int, vdim: int, state: int, groups: int,
+                 conv_taps: int, norm_groups: int, eps: float, conv_bias: bool = True):
+        super().__init__()
+        assert num_heads % groups == 0 and (num_heads * vdim) % norm_groups == 0
+        self.num_heads = num_heads
+        self.vdim = vdim
+        self.state = state
+        self.groups = groups
+        self.norm_groups = norm_groups
+        self.eps = float(eps)
+        self.inner = num_heads * vdim
+        self.conv_channels = self.inner + 2 * groups * state
+        # [z | x B C | dt] widths of the caller's input projection
+        self.splits = [self.inner, self.conv_channels, num_heads]
+        self.conv = CausalShortConv(self.conv_channels, conv_taps, activation="silu",
+                                    bias=conv_bias)
+        f32 = dict(dtype=torch.float32)
+        self.A_log = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False)
+        self.D = nn.Parameter(torch.ones(num_heads, **f32), requires_grad=False)
+        self.norm_weight = nn.Parameter(torch.ones(self.inner, **f32), requires_grad=False)
+
+    def state_shapes(self):
+        return {"conv": self.conv.state_shape(),
+                "ssm": (self.num_heads, self.vdim, self.state)}   # stored transposed
+
+    def forward(self, z: torch.Tensor, xbc: torch.Tensor, dt: torch.Tensor,
+                states, key: str, step: seqmix.StepLayout) -> torch.Tensor:
+        """z (B,S,inner), xbc (B,S,inner + 2*groups*state), dt (B,S,heads):
+        raw projections (column slices of one GEMM output are fine). Returns
+        (B,S,inner) in z's dtype."""
+        GN = self.groups * self.state
+        c = self.conv(xbc, states.get(key + ".conv"), step, out_dtype=torch.float32)
+        x, Bm, Cm = torch.split(c, [self.inner, GN, GN], dim=-1)
+        y = seqmix.decay_scan(Cm, Bm, x, states.get(key + ".ssm"), step, self.state,
+                              self.vdim, dt=dt, dt_bias=self.dt_bias, a_log=self.A_log,
+                              skip=self.D)
+        return seqmix.group_gated_norm(y, z, self.norm_weight, self.eps, self.norm_groups,
+                                       gate_first=True, out_dtype=z.dtype)
+
+
+class Retention(nn.Module):
+    """Linear attention with a fixed decay per head and no softmax or
+    denominator: per head a (dim x vdim) fp32 state
+
+        S_t = decay_h S_{t-1} + (dim^-1/2 k_t) v_t^T ,   o_t = S_t^T q_t ,
+
+    each head's read-out divided by its root mean square (no weight), then
+    multiplied by silu of a gate projection. The caller owns the q/k/v/gate
+    and output projections; the state lives in the cache manager's
+    :class:`RecurrentStateManager`.
+    """
+
+    def __init__(self, num_heads: int, dim: int, vdim: int, decay, eps: float):
+        super().__init__()
+        assert len(decay) == num_heads
+        self.num_heads = num_heads
+        self.dim = dim
+        self.vdim = vdim
+        self.eps = float(eps)
+        self.register_buffer("decay", torch.tensor([float(d) for d in decay],
+                                                   dtype=torch.float32), persistent=False)
+
+    def state_shapes(self):
+        return {"mem": (self.num_heads, self.vdim, self.dim)}      # stored transposed
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
+                states, key: str, step: seqmix.StepLayout) -> torch.Tensor:
+        """q, k (B,S,H*dim), v, gate (B,S,H*vdim). Returns (B,S,H*vdim) in the
+        gate's dtype."""
+        o = seqmix.decay_scan(q, k, v, states.get(key + ".mem"), step, self.dim, self.vdim,
+                              head_decay=self.decay, k_scale=self.dim ** -0.5)
+        return seqmix.group_gated_norm(o, gate, None, self.eps, self.num_heads,
+                                       gate_first=False, out_dtype=gate.dtype)

@@ -394,3 +394,105 @@ class MoELayer(nn.Module):
             out = out + self.shared_expert(flat)
         out = mappings.reduce_from_tensor_parallel_region(out)
         return out.view(B, S, H)
+
+
+class GroupLimitedRouter(nn.Module):
+    """Softmax router whose experts form groups of neighbours: a group scores
+    as its best expert, and only experts of the ``keep_groups`` best groups
+    compete for the ``top_k`` places. The weights are the chosen experts'
+    softmax scores over ALL experts times ``scale`` (renormalised over the
+    chosen ones first when ``normalize``). Logits, softmax and selection are
+    fp32. ``extra_gates`` further rows of the weight are per-token sigmoid
+    gates computed by the same fp32 product (a shared expert's gate)."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int, n_groups: int = 1,
+                 keep_groups: int = 1, scale: float = 1.0, normalize: bool = False,
+                 extra_gates: int = 0):
+        super().__init__()
+        assert num_experts % max(n_groups, 1) == 0 and top_k <= num_experts
+        self.num_experts = num_experts
+        self.top_k = top_k
+        self.n_groups = max(int(n_groups), 1)
+        self.keep_groups = max(min(int(keep_groups), self.n_groups), 1)
+        per = num_experts // self.n_groups
+        assert top_k <= per * self.keep_groups, "top_k exceeds the experts of the kept groups"
+        self.scale = float(scale)
+        self.normalize = bool(normalize)
+        self.weight = nn.Parameter(
+            torch.empty(num_experts + extra_gates, hidden_size, dtype=torch.float32),
+            requires_grad=False)
+
+    def forward(self, x: torch.Tensor):
+        """x (T, hidden) -> (dense (T, E + extra) fp32, idx (T, top_k) int32,
+        weights (T, top_k) fp32)."""
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        logits = F.linear(x.float(), self.weight)
+        return seqmix.group_limited_router(logits, self.num_experts, self.top_k, self.n_groups,
+                                           self.keep_groups, self.scale, self.normalize)
+
+
+class FusedUngatedExperts(nn.Module):
+    """Two-matrix experts ``W_down act(W_up x)`` with act = relu squared,
+    stacked so that ALL experts (and an optional always-on shared expert) are
+    two GEMMs: ``up`` (E*ff + shared_ff, hidden) and ``down`` (hidden, E*ff +
+    shared_ff). The routing weight (zero for an unchosen expert) multiplies
+    the activation before the second product, whose fp32 accumulator then
+    carries the sum over experts. Every expert's weights stream once per step
+    whatever the batch, which is the memory traffic of a decode step anyway;
+    the step has no data-dependent shapes and no host synchronisation."""
+
+    def __init__(self, num_experts: int, hidden_size: int, expert_ff: int, shared_ff: int,
+                 dtype: torch.dtype, tp_degree: int = 1):
+        super().__init__()
+        from neuronx_distributed_inference_amd.parallel.layers import (
+            ColumnParallelLinear,
+            RowParallelLinear,
+        )
+
+        assert tp_degree == 1
+        self.num_experts = num_experts
+        self.expert_ff = expert_ff
+        self.shared_ff = shared_ff
+        inner = num_experts * expert_ff + shared_ff
+        self.up = ColumnParallelLinear(hidden_size, inner, dtype=dtype, tp_degree=1)
+        self.down = RowParallelLinear(inner, hidden_size, dtype=dtype, tp_degree=1)
+
+    @staticmethod
+    def stack_up(ups, shared_up=None):
+        """[(ff, hidden)] * E (+ (shared_ff, hidden)) -> fused up weight."""
+        return torch.cat(list(ups) + ([shared_up] if shared_up is not None else []), dim=0)
+
+    @staticmethod
+    def stack_down(downs, shared_down=None):
+        """[(hidden, ff)] * E (+ (hidden, shared_ff)) -> fused down weight."""
+        return torch.cat(list(downs) + ([shared_down] if shared_down is not None else []), dim=1)
+
+    def forward(self, x: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
+        """x (T, hidden); gates (T, E [+ 1]) fp32 dense routing weights, the
+        last column the shared expert's gate when there is one."""
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        hid = self.up(x)
+        return self.down(seqmix.relu2_scale(hid, gates, self.expert_ff, self.num_experts,
+                                             out_dtype=hid.dtype))
+
+
+class GroupRoutedFeedForward(nn.Module):
+    """Mixture of relu-squared experts behind a :class:`GroupLimitedRouter`,
+    with an optional shared expert that runs for every token and is scaled by
+    a per-token sigmoid gate (``shared_ff`` = 0: none)."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_ff: int,
+                 dtype: torch.dtype, n_groups: int = 1, keep_groups: int = 1,
+                 scale: float = 1.0, normalize: bool = False, shared_ff: int = 0):
+        super().__init__()
+        self.router = GroupLimitedRouter(hidden_size, num_experts, top_k, n_groups, keep_groups,
+                                         scale, normalize, extra_gates=1 if shared_ff else 0)
+        self.experts = FusedUngatedExperts(num_experts, hidden_size, expert_ff, shared_ff, dtype)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        shape = h.shape
+        flat = h.reshape(-1, shape[-1])
+        dense, _, _ = self.router(flat)
+        return self.experts(flat, dense).view(shape)

@@ -161,3 +161,33 @@ def interleaved_inv_freq(base: float, dims: int) -> torch.Tensor:
     table is the closest one to the exact values."""
     i = torch.arange(dims // 2, dtype=torch.float64)
     return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float()
+
+
+def half_split_inv_freq(base: float, dims: int, scaling: Optional[dict] = None):
+    """Frequency table and cos/sin factor for rotary layouts that pair channel
+    i with channel i + dims/2: f_i = base^(-2i/dims), i < dims/2, evaluated in
+    float64 and rounded once.
+
+    ``scaling`` = {factor, original, fast, slow} applies the by-parts
+    length extension: with turns(t) = dims * ln(original / (2 pi t)) /
+    (2 ln base), lo = max(floor(turns(fast)), 0), hi = min(ceil(turns(slow)),
+    dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i
+    turns at f_i / factor * ramp_i + f_i * (1 - ramp_i) (fast pairs keep
+    their frequency, slow pairs are interpolated), and cos and sin are
+    multiplied by 0.1 ln(factor) + 1. Returns (inv_freq fp32 (dims/2,),
+    factor on cos/sin)."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if not scaling:
+        return f.float(), 1.0
+    factor = float(scaling["factor"])
+    original = float(scaling["original"])
+
+    def turns(t):
+        return dims * math.log(original / (2.0 * math.pi * float(t))) / (2.0 * math.log(base))
+
+    lo = max(math.floor(turns(scaling["fast"])), 0)
+    hi = min(math.ceil(turns(scaling["slow"])), dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.float(), 0.1 * math.log(factor) + 1.0

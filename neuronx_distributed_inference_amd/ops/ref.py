@@ -241,11 +241,11 @@ def _masked_tail(tail_row: torch.Tensor, p0: int) -> torch.Tensor:
 
 
 def short_conv(x, w, tail, positions, seq_ids, activation="none",
-               residual=False, out_dtype=torch.float32):
+               residual=False, out_dtype=torch.float32, bias=None):
     """Depthwise causal convolution over time with a carried tail:
-    y_t = sum_j w[:, j] * x_{t-(taps-1)+j}; the last column of `w`
+    y_t = sum_j w[:, j] * x_{t-(taps-1)+j} (+ bias); the last column of `w`
     multiplies the current token. x (B,S,C); w (C,taps); tail
-    (slots, taps-1, C) fp32."""
+    (slots, taps-1, C) fp32; bias (C,) or None."""
     B, S, C = x.shape
     taps = w.shape[1]
     R = taps - 1
@@ -262,6 +262,8 @@ def short_conv(x, w, tail, positions, seq_ids, activation="none",
         acc = torch.zeros(n, C, dtype=torch.float32, device=x.device)
         for j in range(taps):
             acc = acc + wf[:, j] * ext[j:j + n]
+        if bias is not None:
+            acc = acc + bias.float()
         y[b, :n] = acc
     if activation == "silu":
         y = torch.nn.functional.silu(y)
@@ -299,7 +301,8 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
 
 def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
                     window=None, keep_first=0, r1=None, r2=None, gate=None,
-                    softcap=0.0, sink=None, q_temp=None, out_dtype=torch.float32):
+                    softcap=0.0, sink=None, q_temp=None, out_dtype=torch.float32,
+                    gate_per_head=False):
     """Softmax attention of ragged queries against a paged cache, every
     option a parameter. Query at position i sees key j <= i when no window
     is given, else when i-j < window or j < keep_first. Score, in order:
@@ -309,7 +312,8 @@ def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
     (H,) adds exp(sink_h) to the softmax denominator (a key without value).
     ``v_cache`` may be a narrowed view of ``k_cache`` (values stored inside
     the key rows). q (B,S,H,Dk) -> (B,S,H*Dv), optionally times
-    sigmoid(gate)."""
+    sigmoid(gate): gate (B,S,H*Dv), or (B,S,H) with ``gate_per_head`` (one
+    number per head)."""
     B, S, H, Dk = q.shape
     G, Dv = v_cache.shape[2], v_cache.shape[3]
     bs = k_cache.shape[1]
@@ -345,8 +349,10 @@ def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
         else:
             p = torch.nan_to_num(torch.softmax(s, dim=-1))
         out = torch.einsum("bhsl,blhd->bshd", p, v)
+    if gate is not None and gate_per_head:
+        out = out.reshape(B, S, H, Dv) * torch.sigmoid(gate.float()).view(B, S, H, 1)
     out = out.reshape(B, S, H * Dv)
-    if gate is not None:
+    if gate is not None and not gate_per_head:
         out = out * torch.sigmoid(gate.float())
     return out.to(out_dtype)
 
@@ -444,3 +450,147 @@ def clamped_glu(gate: torch.Tensor, up: torch.Tensor, limit: float,
     g = gate.float().clamp(max=limit)
     u = up.float().clamp(-limit, limit)
     return g * torch.sigmoid(alpha * g) * (u + 1.0)
+
+
+def head_norm_rotate(x: torch.Tensor, positions: torch.Tensor, norm_weight, eps: float,
+                     inv_freq, mscale: float = 1.0) -> torch.Tensor:
+    """Per-head RMS norm (weight (C,) shared by the heads; None = no norm)
+    followed by rotary positions in the half-split layout: inside the first
+    2*len(inv_freq) channels of every head, channel i pairs with channel
+    i + len(inv_freq); angle p * inv_freq[i] in fp32, cos and sin times
+    ``mscale``; the other channels pass unchanged (``inv_freq`` None = no
+    rotation). x (B,S,N,C), positions (B,S); returns fp32."""
+    B, S = positions.shape
+    xf = x.float()
+    if norm_weight is not None:
+        xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) * norm_weight.float()
+    if inv_freq is None or inv_freq.numel() == 0:
+        return xf
+    half = inv_freq.numel()
+    ang = positions.clamp(min=0).float().view(B, S, 1, 1) * inv_freq.float()
+    c, sn = torch.cos(ang) * mscale, torch.sin(ang) * mscale
+    u, v = xf[..., :half], xf[..., half:2 * half]
+    return torch.cat([u * c - v * sn, v * c + u * sn, xf[..., 2 * half:]], dim=-1)
+
+
+def decay_scan(q, k, v, state, positions, seq_ids, dim: int, vdim: int,
+               dt=None, dt_bias=None, a_log=None, head_decay=None,
+               k_scale: float = 1.0, skip=None):
+    """Linear recurrence with a scalar decay per head and matrix state,
+    carried in ``state`` (slots, H, vdim, dim) fp32 (stored transposed):
+
+        S_t = a_t S_{t-1} + k_t (w_t v_t)^T ;  o_t = S_t^T q_t (+ skip_h v_t)
+
+    Two ways to give the decay: ``dt`` (B,S,H) raw step-size projections with
+    ``dt_bias`` and ``a_log`` (H,): w_t = softplus(dt + dt_bias), a_t =
+    exp(-exp(a_log) w_t) (selective state spaces: k = B, q = C, v = x); or
+    ``head_decay`` (H,): a_t = head_decay, w_t = 1 (retention). q, k
+    (B,S,G*dim) are shared by H/G consecutive heads, v (B,S,H*vdim); k is
+    multiplied by ``k_scale``. Returns fp32 (B,S,H*vdim)."""
+    B, S = positions.shape
+    D, Dv = dim, vdim
+    H = v.shape[-1] // Dv
+    G = q.shape[-1] // D
+    rep = H // G
+    qf = q.float().reshape(B, S, G, D).repeat_interleave(rep, dim=2)
+    kf = (k.float() * k_scale).reshape(B, S, G, D).repeat_interleave(rep, dim=2)
+    vf = v.float().reshape(B, S, H, Dv)
+    if dt is not None:
+        w = torch.nn.functional.softplus(dt.float() + dt_bias.float(), threshold=20.0)
+        a = torch.exp(-torch.exp(a_log.float()) * w)
+    else:
+        a = head_decay.float().view(1, 1, H).expand(B, S, H)
+        w = torch.ones(B, S, H, dtype=torch.float32, device=v.device)
+    out = torch.zeros(B, S, H, Dv, dtype=torch.float32, device=v.device)
+    n_valid, p0s = _row_extent(positions)
+    for b in range(B):
+        slot = int(seq_ids[b])
+        n = int(n_valid[b])
+        if slot < 0 or n == 0:
+            continue
+        St = state[slot].float().transpose(-1, -2).clone() if int(p0s[b]) > 0 else torch.zeros(
+            H, D, Dv, dtype=torch.float32, device=v.device)
+        for t in range(n):
+            St = a[b, t].view(H, 1, 1) * St + kf[b, t].unsqueeze(-1) * (
+                w[b, t].view(H, 1) * vf[b, t]).unsqueeze(1)
+            out[b, t] = torch.einsum("hdv,hd->hv", St, qf[b, t])
+        state[slot] = St.transpose(-1, -2).to(state.dtype)
+    if skip is not None:
+        out = out + skip.float().view(1, 1, H, 1) * vf
+    return out.reshape(B, S, H * Dv)
+
+
+def group_gated_norm(y, gate, weight, eps: float, groups: int, gate_first: bool,
+                     out_dtype=torch.float32):
+    """RMS norm of (.., C) rows in ``groups`` equal parts (each part by its
+    own root mean square), optional weight (C,), and a silu gate applied
+    before the norm (``gate_first``) or after it."""
+    yf = y.float()
+    g = torch.nn.functional.silu(gate.float())
+    if gate_first:
+        yf = yf * g
+    shp = yf.shape
+    yg = yf.reshape(*shp[:-1], groups, shp[-1] // groups)
+    yf = (yg * torch.rsqrt((yg * yg).mean(-1, keepdim=True) + eps)).reshape(shp)
+    if weight is not None:
+        yf = yf * weight.float()
+    if not gate_first:
+        yf = yf * g
+    return yf.to(out_dtype)
+
+
+def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int,
+                         keep_groups: int, scale: float, normalize: bool = False):
+    """Softmax over the first ``num_experts`` columns of fp32 ``logits``
+    (T, E + extra); experts form ``n_groups`` groups of neighbours, a group
+    scores as its best expert and only experts of the ``keep_groups`` best
+    groups compete for the ``top_k`` places. Weights are the chosen experts'
+    softmax scores times ``scale`` (divided by their sum first when
+    ``normalize``). Extra columns are per-token sigmoid gates. Returns
+    (dense (T, E + extra) fp32 with zeros at unchosen experts, idx (T, top_k)
+    int32, weights (T, top_k) fp32)."""
+    T = logits.shape[0]
+    E = num_experts
+    lf = logits.float()
+    s = torch.softmax(lf[:, :E], dim=-1)
+    cand = s
+    if n_groups > 1 and keep_groups < n_groups:
+        per = E // n_groups
+        gs = s.view(T, n_groups, per).max(-1).values
+        best = gs.topk(keep_groups, dim=-1).indices
+        gmask = torch.zeros_like(gs, dtype=torch.bool).scatter(1, best, True)
+        cand = torch.where(gmask.repeat_interleave(per, dim=1), s, torch.full_like(s, -1.0))
+    idx = cand.topk(top_k, dim=-1).indices
+    w = s.gather(1, idx)
+    if normalize:
+        w = w / w.sum(-1, keepdim=True)
+    w = w * scale
+    dense = torch.zeros_like(lf)
+    dense[:, :E] = torch.zeros_like(s).scatter(1, idx, w)
+    dense[:, E:] = torch.sigmoid(lf[:, E:])
+    return dense, idx.to(torch.int32), w
+
+
+def relu2_scale(hid, gates, expert_ff: int, num_experts: int, out_dtype):
+    """(T, E*ff + rest) hidden pre-activations -> relu(x)^2 times the token's
+    gate of the column's owner: column c < E*ff belongs to expert c // ff,
+    the remaining columns (a shared expert) to gate column E; ``gates`` is
+    (T, E + 1), or (T, E) when there are no remaining columns."""
+    T, C = hid.shape
+    E = num_experts
+    assert C == E * expert_ff or gates.shape[1] == E + 1
+    hf = torch.relu(hid.float()) ** 2
+    cols = (torch.arange(C, device=hid.device) // expert_ff).clamp(max=E)
+    return (hf * gates.float()[:, cols]).to(out_dtype)
+
+
+def scaled_residual(x, terms):
+    """In place on the fp32 stream: x += sum_i f_i(y_i) * w_i with w_i a
+    per-channel vector and f_i the identity or an RMS norm over the row
+    (``terms``: (y, w, eps or None))."""
+    for y, w, eps in terms:
+        yf = y.float()
+        if eps is not None:
+            yf = yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps)
+        x.add_(yf * w.float())
+    return x

@@ -187,9 +187,10 @@ def layer_norm(x, weight, eps: float, out_dtype: torch.dtype):
 
 
 def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
-               residual: bool = False, out_dtype=torch.float32):
-    """Depthwise causal conv over time with a carried tail (see
-    ref.short_conv). Does not advance the tail: call short_conv_commit."""
+               residual: bool = False, out_dtype=torch.float32, bias=None):
+    """Depthwise causal conv over time with a carried tail and an optional
+    per-channel bias (see ref.short_conv). Does not advance the tail: call
+    short_conv_commit."""
     if x.is_cuda:
         lib = _load()
         B, S, C = x.shape
@@ -197,10 +198,11 @@ def short_conv(x, w, tail, step: StepLayout, activation: str = "none",
         _check(lib.nx_short_conv(
             _p(x), ctypes.c_long(_rows_view(x)), _is_bf16(x), _p(_f32(w)), _p(tail), _p(step.positions),
             _p(step.seq_ids), _p(step.nvalid), _p(y), _is_bf16(y), B, S, C, w.shape[1],
-            int(activation == "silu"), int(residual), _stream()), "short_conv")
+            int(activation == "silu"), int(residual),
+            _p(None if bias is None else _f32(bias)), _stream()), "short_conv")
         return y
     return ref.short_conv(x, w, tail, step.positions, step.seq_ids,
-                          activation, residual, out_dtype)
+                          activation, residual, out_dtype, bias)
 
 
 def short_conv_commit(x, tail, step: StepLayout):
@@ -247,12 +249,13 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping, step: "StepLayo
 def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: float,
                     num_heads: int, window: Optional[int] = None, keep_first: int = 0,
                     r1=None, r2=None, gate=None, softcap: float = 0.0, sink=None,
-                    q_temp=None, out_dtype=None):
+                    q_temp=None, out_dtype=None, gate_per_head: bool = False):
     """q (B,S,H*Dk) (row-strided view allowed) against the paged cache ->
     (B,S,H*Dv). Options (see ref.paged_attention): sliding ``window`` with
     ``keep_first`` always-visible tokens (None = plain causal), log-distance
     penalty ``r1``/``r2``, tanh score cap, per-head softmax ``sink``, query
-    temperature ``q_temp`` = (coef, every), sigmoid output ``gate``.
+    temperature ``q_temp`` = (coef, every), sigmoid output ``gate``
+    ((B,S,H*Dv), or (B,S,H) with ``gate_per_head``).
     ``v_cache`` may be ``k_cache[..., :Dv]`` (values inside the key rows)."""
     B, S = q.shape[0], q.shape[1]
     H = num_heads
@@ -291,12 +294,13 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
             k_cache.shape[1], ctypes.c_float(scale),
             int(window) if window is not None else 0x7fffffff, int(keep_first),
             ctypes.c_float(softcap or 0.0), ctypes.c_float(coef), every,
-            _p(ws), nks, _stream()), "paged_attention")
+            _p(ws), nks, int(bool(gate_per_head)), _stream()), "paged_attention")
         return out
     return ref.paged_attention(
         q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table, scale,
         window=window, keep_first=keep_first, r1=r1, r2=r2, gate=gate,
-        softcap=softcap or 0.0, sink=sink, q_temp=q_temp, out_dtype=out_dtype)
+        softcap=softcap or 0.0, sink=sink, q_temp=q_temp, out_dtype=out_dtype,
+        gate_per_head=gate_per_head)
 
 
 def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
@@ -486,3 +490,159 @@ def clamped_glu_fused(gate_up, limit: float, alpha: float = 1.702):
 def scaled_embedding(h, scale: float):
     """Embedding rows -> fp32 residual stream, times a constant."""
     return h.float().mul_(scale) if h.dtype != torch.float32 else h * scale
+
+
+def head_norm_rotate(x, step: StepLayout, norm_weight, eps: float, inv_freq,
+                     mscale: float = 1.0, out_dtype=None):
+    """Per-head RMS norm (weight shared by the heads, None = none) and
+    half-split rotary positions (channel i pairs with i + len(inv_freq), cos
+    and sin times ``mscale``; None = no rotation) in one pass, statistics and
+    angles in fp32. x (B,S,N,C), possibly a strided view of a fused
+    projection; returns a dense (B,S,N*C) tensor."""
+    out_dtype = out_dtype or x.dtype
+    B, S, N, C = x.shape
+    if x.is_cuda:
+        lib = _load()
+        out = torch.empty(B, S, N * C, dtype=out_dtype, device=x.device)
+        assert x.stride(3) == 1
+        half = 0 if inv_freq is None else inv_freq.numel()
+        assert 2 * half <= C
+        _check(lib.nx_head_norm_rope(
+            _p(x), ctypes.c_long(_token_stride(x)), ctypes.c_long(x.stride(2)), _is_bf16(x),
+            _p(out), _is_bf16(out), _p(step.positions),
+            _p(None if norm_weight is None else _f32(norm_weight)), ctypes.c_float(eps),
+            _p(None if half == 0 else _f32(inv_freq)), half, ctypes.c_float(mscale),
+            ctypes.c_long(B * S), N, C, _stream()), "head_norm_rotate")
+        return out
+    return ref.head_norm_rotate(x, step.positions, norm_weight, eps, inv_freq,
+                                mscale).reshape(B, S, N * C).to(out_dtype)
+
+
+def decay_scan(q, k, v, state, step: StepLayout, dim: int, vdim: int, dt=None,
+               dt_bias=None, a_log=None, head_decay=None, k_scale: float = 1.0, skip=None):
+    """Scalar-decay linear recurrence with matrix state (see ref.decay_scan):
+    selective state spaces (``dt``/``dt_bias``/``a_log``) or fixed per-head
+    decays (``head_decay``). q, k (B,S,G*dim), v (B,S,H*vdim) may be column
+    slices of wider tensors; ``state`` (slots, H, vdim, dim) fp32 is read
+    (unless the row starts at position 0) and advanced. Returns fp32."""
+    assert (dt is None) != (head_decay is None)
+    if v.is_cuda:
+        lib = _load()
+        B, S = v.shape[0], v.shape[1]
+        H = v.shape[-1] // vdim
+        G = q.shape[-1] // dim
+        assert q.dtype == k.dtype == v.dtype and state.dtype == torch.float32
+        assert state.is_contiguous() and tuple(state.shape[1:]) == (H, vdim, dim)
+        assert H % G == 0 and q.shape[-1] == G * dim and k.shape[-1] == G * dim
+        out = torch.empty(B, S, H * vdim, dtype=torch.float32, device=v.device)
+        _check(lib.nx_decay_scan(
+            _p(q), ctypes.c_long(_rows_view(q)), _p(k), ctypes.c_long(_rows_view(k)),
+            _p(v), ctypes.c_long(_rows_view(v)), _is_bf16(v),
+            _p(dt), ctypes.c_long(0 if dt is None else _rows_view(dt)),
+            0 if dt is None else _is_bf16(dt),
+            _p(None if dt_bias is None else _f32(dt_bias)),
+            _p(None if a_log is None else _f32(a_log)),
+            _p(None if head_decay is None else _f32(head_decay)),
+            ctypes.c_float(k_scale), _p(None if skip is None else _f32(skip)),
+            _p(state), _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(out),
+            B, S, H, G, dim, vdim, _stream()), "decay_scan")
+        return out
+    return ref.decay_scan(q, k, v, state, step.positions, step.seq_ids, dim, vdim,
+                          dt=dt, dt_bias=dt_bias, a_log=a_log, head_decay=head_decay,
+                          k_scale=k_scale, skip=skip)
+
+
+def group_gated_norm(y, gate, weight, eps: float, groups: int, gate_first: bool,
+                     out_dtype=torch.float32):
+    """RMS norm of fp32 rows in ``groups`` equal parts with a silu gate before
+    or after it and an optional weight (see ref.group_gated_norm). ``gate``
+    may be a column slice of a wider tensor."""
+    if y.is_cuda:
+        lib = _load()
+        C = y.shape[-1]
+        assert y.dtype == torch.float32 and y.is_contiguous() and C % groups == 0
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        _check(lib.nx_group_gated_norm(
+            _p(y), _p(gate), ctypes.c_long(_rows_view(gate)), _is_bf16(gate),
+            _p(None if weight is None else _f32(weight)), ctypes.c_float(eps), groups,
+            int(gate_first), _p(out), _is_bf16(out), ctypes.c_long(y.numel() // C), C,
+            _stream()), "group_gated_norm")
+        return out
+    return ref.group_gated_norm(y, gate, weight, eps, groups, gate_first, out_dtype)
+
+
+def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int = 1,
+                         keep_groups: int = 1, scale: float = 1.0, normalize: bool = False):
+    """Group-limited top-k routing on fp32 logits (T, E + extra) (see
+    ref.group_limited_router): returns (dense (T, E + extra) weights with
+    sigmoid gates in the extra columns, idx (T, top_k) int32, weights)."""
+    if logits.is_cuda:
+        lib = _load()
+        T, C = logits.shape
+        E = num_experts
+        assert logits.dtype == torch.float32 and logits.stride(1) == 1
+        assert E % max(n_groups, 1) == 0 and top_k <= E
+        dense = torch.empty(T, C, dtype=torch.float32, device=logits.device)
+        idx = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
+        wts = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
+        _check(lib.nx_group_router(
+            _p(logits), ctypes.c_long(logits.stride(0)), E, C - E, top_k, max(n_groups, 1),
+            max(min(keep_groups, n_groups), 1), ctypes.c_float(scale), int(normalize),
+            _p(dense), _p(idx), _p(wts), ctypes.c_long(T), _stream()), "group_limited_router")
+        return dense, idx, wts
+    return ref.group_limited_router(logits, num_experts, top_k, max(n_groups, 1),
+                                    max(min(keep_groups, n_groups), 1), scale, normalize)
+
+
+def relu2_scale(hid, gates, expert_ff: int, num_experts: int, out_dtype=None):
+    """relu(x)^2 of (T, E*ff + rest) pre-activations times the token's gate of
+    the column's expert; the remaining columns take gate column E (see
+    ref.relu2_scale)."""
+    out_dtype = out_dtype or hid.dtype
+    if hid.is_cuda:
+        lib = _load()
+        T, C = hid.shape
+        assert hid.is_contiguous() and gates.dtype == torch.float32 and gates.is_contiguous()
+        assert out_dtype == hid.dtype
+        assert C == num_experts * expert_ff or gates.shape[1] == num_experts + 1
+        out = torch.empty(T, C, dtype=out_dtype, device=hid.device)
+        _check(lib.nx_relu2_scale(_p(hid), _is_bf16(hid), _p(gates), gates.shape[1], expert_ff,
+                                  num_experts, _p(out), ctypes.c_long(T), C, _stream()),
+               "relu2_scale")
+        return out
+    return ref.relu2_scale(hid, gates, expert_ff, num_experts, out_dtype)
+
+
+def scaled_residual(x, terms, eps: float = 0.0):
+    """In place on the fp32 stream: x += sum_i f_i(y_i) * w_i for up to three
+    terms (y (..., C) in one dtype, w (C,) fp32, normed): f_i is an RMS norm
+    over the row (with ``eps``) when ``normed`` else the identity."""
+    assert 1 <= len(terms) <= 3
+    if x.is_cuda:
+        lib = _load()
+        C = x.shape[-1]
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        args = []
+        keep = []
+        for i in range(3):
+            if i < len(terms):
+                y, w, normed = terms[i]
+                y = y.contiguous()
+                assert y.dtype == terms[0][0].dtype and y.numel() == x.numel()
+                wf = _f32(w)
+                keep += [y, wf]
+                args += [_p(y), _p(wf), int(bool(normed))]
+            else:
+                args += [_p(None), _p(None), 0]
+        _check(lib.nx_scaled_residual(_p(x), *args, _is_bf16(terms[0][0]), ctypes.c_float(eps),
+                                      ctypes.c_long(x.numel() // C), C, _stream()),
+               "scaled_residual")
+        return x
+    return ref.scaled_residual(x, [(y, w, eps if normed else None) for y, w, normed in terms])
+
+
+def embed_positions(h, pos_table, step: StepLayout):
+    """Token embedding rows (B,S,W) plus a learned position row per token ->
+    fp32 residual stream; pad tokens (position -1) take row 0."""
+    p = step.positions.long().clamp(min=0)
+    return h.float() + pos_table[p].float()

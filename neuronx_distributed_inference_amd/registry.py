@@ -71,6 +71,11 @@ _REGISTRY: Dict[str, Tuple[str, str, str]] = {
         "NabelixInferenceConfig",
         "NabelixForCausalLM",
     ),
+    "kuterax": (
+        "neuronx_distributed_inference_amd.models.kuterax.modeling_kuterax",
+        "KuteraxInferenceConfig",
+        "KuteraxForCausalLM",
+    ),
     "soputar": (
         "neuronx_distributed_inference_amd.models.soputar.modeling_soputar",
         "SoputarInferenceConfig",
