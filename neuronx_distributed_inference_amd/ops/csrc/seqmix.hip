@@ -112,7 +112,8 @@ template <typename TIn, typename TOut>
 __global__ void short_conv_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w,
                                   const float* __restrict__ tail, const int* __restrict__ pos,
                                   const int* __restrict__ seq, TOut* __restrict__ y,
-                                  int B, int S, int C, int taps, int act_silu, int residual) {
+                                  int B, int S, int C, int taps, int act_silu, int residual,
+                                  const float* __restrict__ bias) {
     const long total = (long)B * S * C;
     const int R = taps - 1;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -125,7 +126,7 @@ __global__ void short_conv_kernel(const TIn* __restrict__ x, long xs, const floa
         const int slot = seq[b];
         if (p < 0 || slot < 0) { stf<TOut>(y + idx, 0.f); continue; }
         const float* wr = w + (long)c * taps;
-        float acc = 0.f, cur = 0.f;
+        float acc = bias ? bias[c] : 0.f, cur = 0.f;
         for (int j = 0; j < taps; ++j) {
             const int col = t - R + j;
             float xv;
@@ -163,7 +164,7 @@ __global__ void short_conv_tile_kernel(const TIn* __restrict__ x, long xs,
                                        const int* __restrict__ pos, const int* __restrict__ seq,
                                        const int* __restrict__ nvalid, TOut* __restrict__ y,
                                        int S, int C, int tiles_per_row, int act_silu,
-                                       int residual) {
+                                       int residual, const float* __restrict__ bias) {
     constexpr int R = TAPS - 1;
     const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
     if (c >= C) return;
@@ -178,6 +179,9 @@ __global__ void short_conv_tile_kernel(const TIn* __restrict__ x, long xs,
     for (int e = 0; e < 8; ++e)
 #pragma unroll
         for (int j = 0; j < TAPS; ++j) wr[e][j] = w[(long)(c + e) * TAPS + j];
+    float bs[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) bs[e] = bias ? bias[c + e] : 0.f;
     float hist[R > 0 ? R : 1][8];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -197,9 +201,10 @@ __global__ void short_conv_tile_kernel(const TIn* __restrict__ x, long xs,
             load8<TIn>(x + ((long)b * S + t) * xs + c, cur);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float acc = wr[e][R] * cur[e];
+                float acc = bs[e];
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc += wr[e][r] * hist[r][e];
+                acc += wr[e][R] * cur[e];
                 if (act_silu) acc = acc * sigmoidf_(acc);
                 if (residual) acc += cur[e];
                 o[e] = acc;
@@ -312,7 +317,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                    int bsz, int S, float scale, int window, int keep, int HPW, int QT,
                    int chunks, int lpr, int pws, long ktok, long khead, long vtok, long vhead,
                    int kvec, const float* __restrict__ sink, float cap, float qt_coef,
-                   int qt_every) {
+                   int qt_every, int ghead) {
     // lpr > 0 (decode shape only): P.V with 8 value channels per lane and
     // 64/lpr keys per step, 16-byte V loads; pws = floats of LDS per wave
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -582,7 +587,10 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
             inv = ca / (l_run[r] * ca + expf(rsink[r] - mf));
         }
         TOut* op = out + (tok * H + h) * (long)Dv;
-        const T* gp = gate ? gate + tok * gstride + (long)h * Dv : nullptr;
+        // gate: one number per value channel, or (ghead) one per head
+        const T* gp = gate ? gate + tok * gstride + (ghead ? (long)h : (long)h * Dv) : nullptr;
+        if (gp && ghead) inv *= sigmoidf_(ldf<T>(gp));
+        if (ghead) gp = nullptr;
 #pragma unroll
         for (int c = 0; c < MAXR; ++c) {
             const int d = lane + c * WAVE;
@@ -634,7 +642,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                        long gstride, bf16* __restrict__ out, int H, int G, int Dk, int Dv,
                        int bsz, int S, float scale, int window, int keep, int QT, long ktok,
                        long khead, long vtok, long vhead, const float* __restrict__ sink,
-                       float cap, float qt_coef, int qt_every, int nsplit) {
+                       float cap, float qt_coef, int qt_every, int nsplit, int ghead) {
     constexpr int KB = MA_KT / 16;           // 16-key score blocks per tile
     constexpr int KS = DKP + 8;              // K tile row stride (elements)
     constexpr int VS = MA_KT + 8;            // V^T tile row stride
@@ -906,12 +914,14 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         const int tq = row / rep, h = g * rep + row % rep;
         const long tok = (long)b * S + t0 + tq;
         bf16* op = out + (tok * H + h) * (long)Dv + dv0;
-        const bf16* gp = gate ? gate + tok * gstride + (long)h * Dv + dv0 : nullptr;
+        const bf16* gp = (gate && !ghead) ? gate + tok * gstride + (long)h * Dv + dv0 : nullptr;
+        const float hg = (gate && ghead)
+            ? sigmoidf_(__bfloat162float(gate[tok * gstride + h])) : 1.f;
 #pragma unroll
         for (int nb = 0; nb < DVP / 16; ++nb) {
             const int d = nb * 16 + lr;
             if (d >= dvn) continue;
-            float o = o_acc[nb][r] * inv;
+            float o = o_acc[nb][r] * inv * hg;
             if (gp) o *= sigmoidf_(__bfloat162float(gp[d]));
             op[d] = __float2bfloat16(o);
         }
@@ -1658,6 +1668,352 @@ __global__ void clamped_glu_vec_kernel(const T* __restrict__ gu, T* __restrict__
     }
 }
 
+// ------------------------------------------- per-head norm + half-split rotary
+// One wave per (token, head): RMS norm over the head's C channels with a weight
+// shared by the heads (optional), then rotary positions on the first 2*half
+// channels, channel i paired with channel i + half, angle pos * inv_freq[i],
+// cos and sin times mscale (half = 0: none). Statistics and angles are fp32;
+// the normed row goes through LDS so a lane can read its partner channel.
+#define HN_WAVES 4
+#define HN_MAXC 512
+
+template <typename TIn, typename TOut>
+__global__ void __launch_bounds__(HN_WAVES * WAVE)
+head_norm_rope_kernel(const TIn* __restrict__ x, long xt, long xh, TOut* __restrict__ out,
+                      const int* __restrict__ pos, const float* __restrict__ nw, float eps,
+                      const float* __restrict__ inv_freq, int half, float mscale,
+                      long ntok, int N, int C) {
+    __shared__ float rows[HN_WAVES][HN_MAXC];
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
+    const long id = (long)blockIdx.x * HN_WAVES + wv;
+    if (id >= ntok * N) return;
+    const long tok = id / N;
+    const int hd = id % N;
+    const int p = pos[tok];
+    TOut* op = out + (tok * N + hd) * (long)C;
+    if (p < 0) {
+        for (int c = lane; c < C; c += WAVE) stf<TOut>(op + c, 0.f);
+        return;
+    }
+    const TIn* xp = x + tok * xt + (long)hd * xh;
+    float* row = rows[wv];
+    float ss = 0.f;
+    for (int c = lane; c < C; c += WAVE) {
+        const float v = ldf<TIn>(xp + c);
+        row[c] = v;
+        ss += v * v;
+    }
+    if (nw) {
+        const float inv = 1.f / sqrtf(wave_sum(ss) / C + eps);
+        for (int c = lane; c < C; c += WAVE) row[c] = row[c] * inv * nw[c];
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int c = lane; c < C; c += WAVE) {
+        float o = row[c];
+        if (c < 2 * half) {
+            const int i = c < half ? c : c - half;
+            float sn, cs;
+            sincosf((float)p * inv_freq[i], &sn, &cs);
+            sn *= mscale; cs *= mscale;
+            o = c < half ? o * cs - row[c + half] * sn : o * cs + row[c - half] * sn;
+        }
+        stf<TOut>(op + c, o);
+    }
+}
+
+// ----------------------------------------------- scalar-decay linear recurrence
+// S_t = a_t S_{t-1} + k_t (w_t v_t)^T, o_t = S_t^T q_t (+ skip_h v_t), one scalar
+// decay per head and token. Workgroup = (row, head, 16 value channels); the 16
+// lanes of a channel split its key rows (lane p owns rows p, p+16, ...), the
+// state sits in registers for the whole step and is read/written once. Tokens
+// are staged through LDS in chunks of DS_TC (q, k, v, decay, step size), so
+// global loads are coalesced and the serial loop reads only LDS.
+// Decay: selective (dt projection + dt_bias, a_log: w = softplus(dt + bias),
+// a = exp(-exp(a_log) w)) or fixed per head (head_decay: a = decay, w = 1).
+#define DS_TC 16
+
+template <typename T, typename TD, int R>
+__global__ void __launch_bounds__(256)
+decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, long ks,
+                  const T* __restrict__ v, long vs, const TD* __restrict__ dt, long dts,
+                  const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                  const float* __restrict__ head_decay, float k_scale,
+                  const float* __restrict__ skip, float* __restrict__ state,
+                  const int* __restrict__ pos, const int* __restrict__ seq,
+                  const int* __restrict__ nvalid, float* __restrict__ out, int S, int H, int G,
+                  int D, int Dv) {
+    constexpr int DP = 16 * R;
+    __shared__ float sq[DS_TC][DP], sk[DS_TC][DP], sv[DS_TC][16], sa[DS_TC], sw[DS_TC];
+    const int b = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * 16;
+    const int slot = seq[b];
+    const int n = slot < 0 ? 0 : nvalid[b];
+    if (n <= 0) return;                                   // uniform
+    const int tid = threadIdx.x, part = tid & 15, cl = tid >> 4;
+    const int c = c0 + cl;
+    const bool cok = c < Dv;
+    const int g = h / (H / G);
+    const int p0 = pos[(long)b * S];
+    float* sp = state + (((long)slot * H + h) * Dv + (cok ? c : 0)) * (long)D;
+    float st[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int d = part + 16 * r;
+        st[r] = (cok && d < D && p0 > 0) ? sp[d] : 0.f;
+    }
+    const float skp = skip ? skip[h] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += DS_TC) {
+        const int cnt = min(DS_TC, n - t0);
+        __syncthreads();                                  // the previous chunk is consumed
+        for (int idx = tid; idx < DS_TC * DP; idx += 256) {
+            const int tt = idx / DP, d = idx % DP;
+            float qv = 0.f, kv = 0.f;
+            if (tt < cnt && d < D) {
+                const long tok = (long)b * S + t0 + tt;
+                qv = ldf<T>(q + tok * qs + (long)g * D + d);
+                kv = ldf<T>(k + tok * ks + (long)g * D + d) * k_scale;
+            }
+            sq[tt][d] = qv;
+            sk[tt][d] = kv;
+        }
+        {
+            const int tt = tid >> 4, cc = tid & 15;       // 256 = DS_TC * 16
+            float vv = 0.f;
+            if (tt < cnt && c0 + cc < Dv)
+                vv = ldf<T>(v + ((long)b * S + t0 + tt) * vs + (long)h * Dv + c0 + cc);
+            sv[tt][cc] = vv;
+        }
+        if (tid < cnt) {
+            float a, w = 1.f;
+            if (dt) {
+                w = softplusf_(ldf<TD>(dt + ((long)b * S + t0 + tid) * dts + h) + dt_bias[h]);
+                a = expf(-expf(a_log[h]) * w);
+            } else {
+                a = head_decay[h];
+            }
+            sa[tid] = a;
+            sw[tid] = w;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < cnt; ++tt) {
+            const float a = sa[tt], xv = sv[tt][cl];
+            const float wv = sw[tt] * xv;
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int d = part + 16 * r;
+                st[r] = a * st[r] + sk[tt][d] * wv;
+                acc += st[r] * sq[tt][d];
+            }
+            acc += __shfl_xor(acc, 8, WAVE);
+            acc += __shfl_xor(acc, 4, WAVE);
+            acc += __shfl_xor(acc, 2, WAVE);
+            acc += __shfl_xor(acc, 1, WAVE);
+            if (part == 0 && cok)
+                out[(((long)b * S + t0 + tt) * H + h) * (long)Dv + c] = acc + skp * xv;
+        }
+    }
+    if (cok) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int d = part + 16 * r;
+            if (d < D) sp[d] = st[r];
+        }
+    }
+}
+
+// ------------------------------------------------ grouped RMS norm with silu gate
+// One wave per (row, group of C/groups channels): y (fp32) is multiplied by
+// silu(gate) before the norm (gate_first) or after it; optional weight.
+template <typename TG, typename TOut>
+__global__ void group_gated_norm_kernel(const float* __restrict__ y, const TG* __restrict__ gate,
+                                        long gs, const float* __restrict__ w, float eps,
+                                        int groups, int gate_first, TOut* __restrict__ out,
+                                        long rows, int C) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long id = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (id >= rows * groups) return;
+    const long row = id / groups;
+    const int gi = id % groups, Cg = C / groups;
+    const float* yp = y + row * C + (long)gi * Cg;
+    const TG* gp = gate + row * gs + (long)gi * Cg;
+    const float* wp = w ? w + (long)gi * Cg : nullptr;
+    TOut* op = out + row * C + (long)gi * Cg;
+    float ss = 0.f;
+    for (int c = lane; c < Cg; c += WAVE) {
+        float v = yp[c];
+        if (gate_first) { const float gv = ldf<TG>(gp + c); v *= gv * sigmoidf_(gv); }
+        ss += v * v;
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / Cg + eps);
+    for (int c = lane; c < Cg; c += WAVE) {
+        const float gv = ldf<TG>(gp + c);
+        const float sg = gv * sigmoidf_(gv);
+        float v = yp[c];
+        if (gate_first) v *= sg;
+        v *= inv;
+        if (wp) v *= wp[c];
+        if (!gate_first) v *= sg;
+        stf<TOut>(op + c, v);
+    }
+}
+
+// ------------------------------------------------------- group-limited router
+// One wave per token: softmax over E logits (fp32), group score = best expert of
+// the group, `keep` best groups stay, `top` best experts among them are chosen
+// (ties: lowest index). Writes the dense (T, E + extra) weight row (zeros at
+// unchosen experts, sigmoid gates in the extra columns), the chosen indices and
+// their weights = score * scale (renormalised over the chosen first if asked).
+DEV void wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, WAVE);
+        const int oi = __shfl_xor(i, o, WAVE);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+#define RT_WAVES 4
+__global__ void __launch_bounds__(RT_WAVES * WAVE)
+group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra, int top,
+                    int ngroups, int keep, float scale, int normalize,
+                    float* __restrict__ dense, int* __restrict__ idx, float* __restrict__ wts,
+                    long T) {
+    extern __shared__ float rsm[];                        // per wave: E scores + ngroups
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
+    const long t = (long)blockIdx.x * RT_WAVES + wv;
+    if (t >= T) return;
+    float* cand = rsm + (long)wv * (E + ngroups);
+    float* gsc = cand + E;
+    const float* lp = logits + t * ls;
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += WAVE) m = fmaxf(m, lp[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += WAVE) { const float x = expf(lp[e] - m); cand[e] = x; sum += x; }
+    sum = wave_sum(sum);
+    const float rs = 1.f / sum;
+    float* dp = dense + t * (long)(E + extra);
+    for (int e = lane; e < E; e += WAVE) { cand[e] *= rs; dp[e] = 0.f; }
+    for (int x = lane; x < extra; x += WAVE) dp[E + x] = sigmoidf_(lp[E + x]);
+    __builtin_amdgcn_wave_barrier();
+    const int per = E / ngroups;
+    if (ngroups > 1 && keep < ngroups) {
+        for (int gi = lane; gi < ngroups; gi += WAVE) {
+            float gm = -1.f;
+            for (int j = 0; j < per; ++j) gm = fmaxf(gm, cand[gi * per + j]);
+            gsc[gi] = gm;
+        }
+        __builtin_amdgcn_wave_barrier();
+        for (int r = 0; r < keep; ++r) {
+            float bv = -2.f; int bi = 0x7fffffff;
+            for (int gi = lane; gi < ngroups; gi += WAVE) {
+                const float x = gsc[gi];
+                if (x <= 1.5f && (x > bv)) { bv = x; bi = gi; }
+            }
+            wave_argmax(bv, bi);
+            if (lane == 0) gsc[bi] = 2.f;                 // kept (scores are <= 1)
+            __builtin_amdgcn_wave_barrier();
+        }
+        for (int e = lane; e < E; e += WAVE) if (gsc[e / per] != 2.f) cand[e] = -1.f;
+        __builtin_amdgcn_wave_barrier();
+    }
+    float wsum = 0.f;
+    float myw = 0.f; int myi = 0;                         // lane r keeps the r-th choice
+    for (int r = 0; r < top; ++r) {
+        float bv = -2.f; int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += WAVE) {
+            const float x = cand[e];
+            if (x > bv) { bv = x; bi = e; }
+        }
+        wave_argmax(bv, bi);
+        if (lane == 0) cand[bi] = -3.f;
+        if (lane == (r & (WAVE - 1))) {
+            // more than 64 choices: flush the previous one first
+            if (r >= WAVE) { idx[t * top + r - WAVE] = myi; wts[t * top + r - WAVE] = myw; }
+            myw = bv; myi = bi;
+        }
+        wsum += bv;
+        __builtin_amdgcn_wave_barrier();
+    }
+    const float f = normalize ? scale / wsum : scale;
+    if (top <= WAVE) {
+        if (lane < top) {
+            idx[t * top + lane] = myi;
+            wts[t * top + lane] = myw * f;
+            dp[myi] = myw * f;
+        }
+    }
+}
+
+// -------------------------------------------------- relu^2 times routing weight
+// out[t, c] = relu(x[t, c])^2 * gates[t, min(c / ff, E)]
+template <typename T>
+__global__ void relu2_scale_kernel(const T* __restrict__ x, const float* __restrict__ gates,
+                                   int gcols, int ff, int E, T* __restrict__ out, long rows,
+                                   int C) {
+    const long total = rows * C;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C;
+        const int c = i % C;
+        const int e = min(c / ff, E);
+        const float v = fmaxf(ldf<T>(x + i), 0.f);
+        stf<T>(out + i, v * v * gates[t * gcols + e]);
+    }
+}
+
+template <typename T>
+__global__ void relu2_scale_vec_kernel(const T* __restrict__ x, const float* __restrict__ gates,
+                                       int gcols, int ff, int E, T* __restrict__ out, long rows,
+                                       int C) {
+    const int C8 = C / 8;
+    const long total = rows * C8;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C8;
+        const int c = (i % C8) * 8;
+        const float gw = gates[t * gcols + min(c / ff, E)];
+        float v[8];
+        load8<T>(x + t * C + c, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { const float r = fmaxf(v[e], 0.f); v[e] = r * r * gw; }
+        store8<T>(out + t * C + c, v);
+    }
+}
+
+// ------------------------------------- residual sum of weighted, optionally normed terms
+// x[row] += sum_i f_i(y_i[row]) * w_i, f_i = RMS norm over the row or identity.
+// One workgroup per row; statistics fp32.
+template <typename T>
+__global__ void __launch_bounds__(LN_THREADS)
+scaled_residual_kernel(float* __restrict__ x, const T* __restrict__ y0,
+                       const float* __restrict__ w0, int n0, const T* __restrict__ y1,
+                       const float* __restrict__ w1, int n1, const T* __restrict__ y2,
+                       const float* __restrict__ w2, int n2, float eps, int C) {
+    __shared__ float red[LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const T* ys[3] = {y0, y1, y2};
+    const float* ws[3] = {w0, w1, w2};
+    const int ns[3] = {n0, n1, n2};
+    float inv[3] = {1.f, 1.f, 1.f};
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        if (!ys[i] || !ns[i]) continue;                   // uniform
+        const T* yr = ys[i] + row * C;
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < C; c += LN_THREADS) { const float v = ldf<T>(yr + c); ss += v * v; }
+        inv[i] = 1.f / sqrtf(block_sum(ss, red) / C + eps);
+    }
+    float* xr = x + row * C;
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+            if (ys[i]) acc += ldf<T>(ys[i] + row * C + c) * inv[i] * ws[i][c];
+        xr[c] += acc;
+    }
+}
+
 // =================================================================== C ABI
 static inline int grid_for(long total, int block, int cap = 8192) {
     long g = (total + block - 1) / block;
@@ -1678,7 +2034,8 @@ int nx_layer_norm(const float* x, const float* w, void* out, int out_bf16, long 
 
 int nx_short_conv(const void* x, long xs, int x_bf16, const float* w, const float* tail,
                   const int* pos, const int* seq, const int* nvalid, void* y, int y_bf16, int B,
-                  int S, int C, int taps, int act_silu, int residual, hipStream_t st) {
+                  int S, int C, int taps, int act_silu, int residual, const float* bias,
+                  hipStream_t st) {
     const long total = (long)B * S * C;
     if (total <= 0) return 0;
     {
@@ -1691,7 +2048,7 @@ int nx_short_conv(const void* x, long xs, int x_bf16, const float* w, const floa
         if (ok) {
             dim3 gt((C / 8 + 127) / 128, (unsigned)(B * tiles)), bt(128);
 #define SCT(TI, TO, TP) short_conv_tile_kernel<TI, TO, TP><<<gt, bt, 0, st>>>( \
-        (const TI*)x, xs, w, tail, pos, seq, nvalid, (TO*)y, S, C, tiles, act_silu, residual)
+        (const TI*)x, xs, w, tail, pos, seq, nvalid, (TO*)y, S, C, tiles, act_silu, residual, bias)
 #define SCTT(TI, TO) do { if (taps == 2) SCT(TI, TO, 2); else if (taps == 3) SCT(TI, TO, 3); \
                           else SCT(TI, TO, 4); } while (0)
             if (x_bf16 && y_bf16) SCTT(bf16, bf16);
@@ -1705,7 +2062,7 @@ int nx_short_conv(const void* x, long xs, int x_bf16, const float* w, const floa
     }
     dim3 grid(grid_for(total, 256)), block(256);
 #define SC(TI, TO) short_conv_kernel<TI, TO><<<grid, block, 0, st>>>( \
-        (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual)
+        (const TI*)x, xs, w, tail, pos, seq, (TO*)y, B, S, C, taps, act_silu, residual, bias)
     if (x_bf16 && y_bf16) SC(bf16, bf16);
     else if (x_bf16) SC(bf16, float);
     else if (y_bf16) SC(float, bf16);
@@ -1748,7 +2105,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
                   const float* sink, const void* gate, long gstride, void* out, int io_bf16,
                   int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
                   float scale, int window, int keep, float cap, float qt_coef, int qt_every,
-                  float* ws, int nks, hipStream_t st) {
+                  float* ws, int nks, int ghead, hipStream_t st) {
     if ((long)B * S <= 0) return 0;
     if (Dv > WAVE * 8 || H % G != 0 || Dk <= 0 || Dv <= 0) return -1;
     if (!io_bf16 && out_bf16) return -2;
@@ -1812,7 +2169,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
 #define MA(DKV, DVV, KTV) paged_attn_mfma_kernel<DKV, DVV, KTV, (KTV == 32)><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
         r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, Dk, Dv, bsz, S, scale, window, \
-        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit)
+        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit, ghead)
 #define MAV(DKV) do { if (dvp == 32) MA(DKV, 32, 64); else if (dvp == 64) MA(DKV, 64, 64); \
                       else if (dvp == 96) MA(DKV, 96, 64); else MA(DKV, 128, 64); } while (0)
             if (wide) {
@@ -1866,7 +2223,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
     window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
-        chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every)
+        chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every, ghead)
 #define WAS(T, TO, MR) do { if (dec) { WA(T, TO, MR, 4, 16); } else { WA(T, TO, MR, 16, 4); } } while (0)
 #define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else if (Dv <= 4 * WAVE) WAS(T, TO, 4); \
                         else WAS(T, TO, 8); } while (0)
@@ -2028,6 +2385,114 @@ int nx_clamped_glu(const void* gu, void* out, int is_bf16, long rows, int I, flo
         (const bf16*)gu, (bf16*)out, rows, I, limit, alpha);
     else clamped_glu_kernel<float><<<grid, block, 0, st>>>(
         (const float*)gu, (float*)out, rows, I, limit, alpha);
+    return (int)hipGetLastError();
+}
+
+int nx_head_norm_rope(const void* x, long xt, long xh, int x_bf16, void* out, int out_bf16,
+                      const int* pos, const float* nw, float eps, const float* inv_freq,
+                      int half, float mscale, long ntok, int N, int C, hipStream_t st) {
+    if (ntok * N <= 0) return 0;
+    if (C > HN_MAXC || 2 * half > C || (half > 0 && !inv_freq)) return -1;
+    const long waves = ntok * N;
+    dim3 grid((unsigned)((waves + HN_WAVES - 1) / HN_WAVES)), block(HN_WAVES * WAVE);
+#define HN(TI, TO) head_norm_rope_kernel<TI, TO><<<grid, block, 0, st>>>( \
+        (const TI*)x, xt, xh, (TO*)out, pos, nw, eps, inv_freq, half, mscale, ntok, N, C)
+    if (x_bf16 && out_bf16) HN(bf16, bf16);
+    else if (x_bf16) HN(bf16, float);
+    else if (out_bf16) HN(float, bf16);
+    else HN(float, float);
+#undef HN
+    return (int)hipGetLastError();
+}
+
+int nx_decay_scan(const void* q, long qs, const void* k, long ks, const void* v, long vs,
+                  int in_bf16, const void* dt, long dts, int dt_bf16, const float* dt_bias,
+                  const float* a_log, const float* head_decay, float k_scale, const float* skip,
+                  float* state, const int* pos, const int* seq, const int* nvalid, float* out,
+                  int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
+    if ((long)B * S <= 0) return 0;
+    if (D <= 0 || Dv <= 0 || G <= 0 || H % G != 0 || D > 256) return -1;
+    if ((dt == nullptr) == (head_decay == nullptr)) return -2;
+    if (dt && (!dt_bias || !a_log)) return -2;
+    if (H > 65535 || B > 65535) return -3;
+    dim3 grid((Dv + 15) / 16, H, B), block(256);
+#define DSK(T, TD, RV) decay_scan_kernel<T, TD, RV><<<grid, block, 0, st>>>( \
+        (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, (const TD*)dt, dts, dt_bias, a_log, \
+        head_decay, k_scale, skip, state, pos, seq, nvalid, out, S, H, G, D, Dv)
+#define DSR(T, TD) do { if (D <= 16) DSK(T, TD, 1); else if (D <= 32) DSK(T, TD, 2); \
+        else if (D <= 64) DSK(T, TD, 4); else if (D <= 128) DSK(T, TD, 8); \
+        else DSK(T, TD, 16); } while (0)
+    if (in_bf16) { if (dt_bf16) DSR(bf16, bf16); else DSR(bf16, float); }
+    else { if (dt_bf16) DSR(float, bf16); else DSR(float, float); }
+#undef DSR
+#undef DSK
+    return (int)hipGetLastError();
+}
+
+int nx_group_gated_norm(const float* y, const void* gate, long gs, int gate_bf16, const float* w,
+                        float eps, int groups, int gate_first, void* out, int out_bf16,
+                        long rows, int C, hipStream_t st) {
+    if (rows <= 0) return 0;
+    if (groups <= 0 || C % groups != 0) return -1;
+    const long waves = rows * groups;
+    dim3 grid((unsigned)((waves + 3) / 4)), block(4 * WAVE);
+#define GN(TG, TO) group_gated_norm_kernel<TG, TO><<<grid, block, 0, st>>>( \
+        y, (const TG*)gate, gs, w, eps, groups, gate_first, (TO*)out, rows, C)
+    if (gate_bf16 && out_bf16) GN(bf16, bf16);
+    else if (gate_bf16) GN(bf16, float);
+    else if (out_bf16) GN(float, bf16);
+    else GN(float, float);
+#undef GN
+    return (int)hipGetLastError();
+}
+
+int nx_group_router(const float* logits, long ls, int E, int extra, int top, int ngroups,
+                    int keep, float scale, int normalize, float* dense, int* idx, float* wts,
+                    long T, hipStream_t st) {
+    if (T <= 0) return 0;
+    if (E <= 0 || top <= 0 || top > E || top > WAVE || ngroups <= 0 || E % ngroups != 0 ||
+        keep <= 0 || keep > ngroups || (long)top > (long)(E / ngroups) * keep) return -1;
+    const size_t sh = (size_t)RT_WAVES * (E + ngroups) * sizeof(float);
+    if (sh > 60 * 1024) return -2;
+    dim3 grid((unsigned)((T + RT_WAVES - 1) / RT_WAVES)), block(RT_WAVES * WAVE);
+    group_router_kernel<<<grid, block, sh, st>>>(logits, ls, E, extra, top, ngroups, keep, scale,
+                                                 normalize, dense, idx, wts, T);
+    return (int)hipGetLastError();
+}
+
+int nx_relu2_scale(const void* x, int is_bf16, const float* gates, int gcols, int ff, int E,
+                   void* out, long rows, int C, hipStream_t st) {
+    if (rows * C <= 0) return 0;
+    if (ff <= 0 || gcols < E || (C > E * ff && gcols < E + 1)) return -1;
+    const int esz = is_bf16 ? 2 : 4;
+    const bool vec = (C % 8) == 0 && (ff % 8) == 0 && ((uintptr_t)x % 16) == 0 &&
+                     ((uintptr_t)out % 16) == 0 && esz > 0;
+    if (vec) {
+        dim3 grid(grid_for(rows * (C / 8), 256)), block(256);
+        if (is_bf16) relu2_scale_vec_kernel<bf16><<<grid, block, 0, st>>>(
+            (const bf16*)x, gates, gcols, ff, E, (bf16*)out, rows, C);
+        else relu2_scale_vec_kernel<float><<<grid, block, 0, st>>>(
+            (const float*)x, gates, gcols, ff, E, (float*)out, rows, C);
+    } else {
+        dim3 grid(grid_for(rows * C, 256)), block(256);
+        if (is_bf16) relu2_scale_kernel<bf16><<<grid, block, 0, st>>>(
+            (const bf16*)x, gates, gcols, ff, E, (bf16*)out, rows, C);
+        else relu2_scale_kernel<float><<<grid, block, 0, st>>>(
+            (const float*)x, gates, gcols, ff, E, (float*)out, rows, C);
+    }
+    return (int)hipGetLastError();
+}
+
+int nx_scaled_residual(float* x, const void* y0, const float* w0, int n0, const void* y1,
+                       const float* w1, int n1, const void* y2, const float* w2, int n2,
+                       int is_bf16, float eps, long rows, int C, hipStream_t st) {
+    if (rows <= 0) return 0;
+    if (!y0 || !w0 || (y1 && !w1) || (y2 && !w2)) return -1;
+    dim3 grid((unsigned)rows), block(LN_THREADS);
+    if (is_bf16) scaled_residual_kernel<bf16><<<grid, block, 0, st>>>(
+        x, (const bf16*)y0, w0, n0, (const bf16*)y1, w1, n1, (const bf16*)y2, w2, n2, eps, C);
+    else scaled_residual_kernel<float><<<grid, block, 0, st>>>(
+        x, (const float*)y0, w0, n0, (const float*)y1, w1, n1, (const float*)y2, w2, n2, eps, C);
     return (int)hipGetLastError();
 }
 
