@@ -1863,6 +1863,8 @@ __global__ void group_gated_norm_kernel(const float* __restrict__ y, const TG* _
 // (ties: lowest index). Writes the dense (T, E + extra) weight row (zeros at
 // unchosen experts, sigmoid gates in the extra columns), the chosen indices and
 // their weights = score * scale (renormalised over the chosen first if asked).
+// A row whose logits are not numbers (the garbage of a pad token) selects the
+// first experts with weight zero: every index stays in range.
 DEV void wave_argmax(float& v, int& i) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -1911,6 +1913,7 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
                 if (x <= 1.5f && (x > bv)) { bv = x; bi = gi; }
             }
             wave_argmax(bv, bi);
+            if ((unsigned)bi >= (unsigned)ngroups) bi = r;   // a row of NaNs compares false everywhere
             if (lane == 0) gsc[bi] = 2.f;                 // kept (scores are <= 1)
             __builtin_amdgcn_wave_barrier();
         }
@@ -1926,6 +1929,7 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
             if (x > bv) { bv = x; bi = e; }
         }
         wave_argmax(bv, bi);
+        if ((unsigned)bi >= (unsigned)E) { bi = r; bv = 0.f; }   // NaN row (a pad token): any valid index
         if (lane == 0) cand[bi] = -3.f;
         if (lane == (r & (WAVE - 1))) {
             // more than 64 choices: flush the previous one first

@@ -337,6 +337,22 @@ def test_group_limited_router_op(device, E, top, count, keep, extra):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_router_rows_that_are_not_numbers(device):
+    """Pad tokens carry garbage: such a row must stay inside its own memory
+    and leave the other rows alone."""
+    torch.manual_seed(5)
+    E, T = 12, 9
+    logits = torch.randn(T, E + 1) * 3
+    clean = seqmix.group_limited_router(logits.to(device), E, 4, 4, 3, 1.0)
+    logits[2] = float("nan")
+    logits[7, 3] = float("inf")
+    dense, idx, wts = seqmix.group_limited_router(logits.to(device), E, 4, 4, 3, 1.0)
+    ok = [0, 1, 3, 4, 5, 6, 8]
+    assert torch.equal(dense[ok].cpu(), clean[0][ok].cpu())
+    assert int(idx.min()) >= 0 and int(idx.max()) < E
+
+
+@pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("E,ff,rest", [(3, 5, 0), (4, 8, 16), (2, 12, 7)])   # scalar / 8-wide
 def test_relu2_scale_op(device, E, ff, rest):
     torch.manual_seed(6)
