@@ -71,9 +71,11 @@ def parse_args():
     p.add_argument("--hybrid", action="store_true",
                    help="prefill/decode throughput of the hybrid decoders (Nabelix: windowed "
                         "attention + gated delta rule; Soputar: latent, delta-rule and capped "
-                        "attention layers) beside Llama at equal width/depth/ff/vocab")
-    p.add_argument("--hybrid-models", default="llama,nabelix,soputar",
-                   help="comma-separated subset of llama,nabelix,soputar for --hybrid")
+                        "attention layers; Kuterax: sink attention + state space in "
+                        "parallel, retention, routed experts) beside Llama at equal "
+                        "width/depth/ff/vocab")
+    p.add_argument("--hybrid-models", default="llama,nabelix,soputar,kuterax",
+                   help="comma-separated subset of llama,nabelix,soputar,kuterax for --hybrid")
     p.add_argument("--hybrid-sizes", default="2048,4096",
                    help="comma-separated layer widths for --hybrid")
     p.add_argument("--hybrid-layers", type=int, default=4)
@@ -109,6 +111,9 @@ def run_hybrid_bench(args):
     )
     from neuronx_distributed_inference_amd.models.soputar.modeling_soputar import (
         SoputarForCausalLM, SoputarInferenceConfig,
+    )
+    from neuronx_distributed_inference_amd.models.kuterax.modeling_kuterax import (
+        KuteraxForCausalLM, KuteraxInferenceConfig,
     )
 
     dtype = "bfloat16" if on_gpu else "float32"
@@ -165,6 +170,28 @@ def run_hybrid_bench(args):
                 neuron_config=ec, architecture="Soputar", width=width, vocab=V,
                 layers=layers, norm={"eps": 1e-5}, embedding={"scale": 8.0})
             cls = SoputarForCausalLM
+        elif kind == "kuterax":
+            # alternating parallel (sink attention + state space) and retention
+            # layers; the feed-forward activates ff columns per token: four of
+            # sixteen experts of ff/8 plus a shared expert of ff/2
+            mlp = {"kind": "moe", "expert": {"ff": ff // 8}, "shared": {"ff": ff // 2},
+                   "router": {"experts": 16, "top": 4, "scale": 2.5,
+                              "groups": {"count": 4, "keep": 2}}}
+            par = {"type": "parallel", "mlp": mlp, "mixer": {
+                "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,
+                         "scale": 128 ** -0.5, "mask": {"size": 1024},
+                         "rot": {"base": 500000.0, "dims": 64, "scaling": {
+                             "factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+                "right": {"heads": 2 * H, "vdim": 64, "state": 128, "groups": G, "conv": 4,
+                          "norm_groups": G}}}
+            ret = {"type": "retention", "mlp": mlp, "mixer": {
+                "heads": H, "dim": 128, "vdim": 128,
+                "decay": [1.0 - 2.0 ** (-5 - (i % 4)) for i in range(H)]}}
+            cfg = KuteraxInferenceConfig(
+                neuron_config=ec, architecture="Kuterax", width=width, vocab=V,
+                max_positions=max_len, layers=[par if i % 2 == 0 else ret for i in range(L)],
+                loop={"start": 0, "stop": L, "times": 1}, norm={"eps": 1e-5})
+            cls = KuteraxForCausalLM
         else:
             layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff}, "mixer": {
                 "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,
@@ -192,7 +219,7 @@ def run_hybrid_bench(args):
         return m
 
     for width in [int(x) for x in args.hybrid_sizes.split(",")]:
-        for kind in [k for k in ("llama", "nabelix", "soputar")
+        for kind in [k for k in ("llama", "nabelix", "soputar", "kuterax")
                      if k in args.hybrid_models.split(",")]:
             with torch.inference_mode():
                 # ---- prefill: one prompt, three timed repetitions

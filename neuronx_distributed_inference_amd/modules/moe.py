@@ -419,8 +419,7 @@ class GroupLimitedRouter(nn.Module):
         self.scale = float(scale)
         self.normalize = bool(normalize)
         self.weight = nn.Parameter(
-            torch.empty(num_experts + extra_gates, hidden_size, dtype=torch.float32),
-            requires_grad=False)
+            torch.empty(num_experts + extra_gates, hidden_size, dtype=torch.float32))
 
     def forward(self, x: torch.Tensor):
         """x (T, hidden) -> (dense (T, E + extra) fp32, idx (T, top_k) int32,

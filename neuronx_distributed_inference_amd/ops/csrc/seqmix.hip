@@ -1730,9 +1730,19 @@ head_norm_rope_kernel(const TIn* __restrict__ x, long xt, long xh, TOut* __restr
 // global loads are coalesced and the serial loop reads only LDS.
 // Decay: selective (dt projection + dt_bias, a_log: w = softplus(dt + bias),
 // a = exp(-exp(a_log) w)) or fixed per head (head_decay: a = decay, w = 1).
+//
+// Long rows with few workgroups are cut into `nseg` segments of `seglen`
+// tokens that run side by side; the recurrence is linear in the state, so
+//   MODE 1: every segment scans from a ZERO state and leaves its end state E_c
+//           and the product P_c of its decays in the workspace (no outputs);
+//   decay_scan_link_kernel: start state of segment c, serially over the few
+//           segments: S_c = P_{c-1} S_{c-1} + E_{c-1} (S_0 = the carried state);
+//   MODE 2: every segment scans again from its true start state and writes
+//           the outputs; the last one stores the carried state.
+// MODE 0 is the plain single pass (decode steps, short portions, full batches).
 #define DS_TC 16
 
-template <typename T, typename TD, int R>
+template <typename T, typename TD, int R, int MODE>
 __global__ void __launch_bounds__(256)
 decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, long ks,
                   const T* __restrict__ v, long vs, const TD* __restrict__ dt, long dts,
@@ -1741,10 +1751,14 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
                   const float* __restrict__ skip, float* __restrict__ state,
                   const int* __restrict__ pos, const int* __restrict__ seq,
                   const int* __restrict__ nvalid, float* __restrict__ out, int S, int H, int G,
-                  int D, int Dv) {
+                  int D, int Dv, float* __restrict__ ws, float* __restrict__ wdec, int nseg,
+                  int seglen) {
     constexpr int DP = 16 * R;
-    __shared__ float sq[DS_TC][DP], sk[DS_TC][DP], sv[DS_TC][16], sa[DS_TC], sw[DS_TC];
-    const int b = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * 16;
+    __shared__ float sq[MODE == 1 ? 1 : DS_TC][DP], sk[DS_TC][DP], sv[DS_TC][16], sa[DS_TC],
+        sw[DS_TC];
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int sgi = MODE == 0 ? 0 : blockIdx.x % nseg;
+    const int c0 = (MODE == 0 ? blockIdx.x : blockIdx.x / nseg) * 16;
     const int slot = seq[b];
     const int n = slot < 0 ? 0 : nvalid[b];
     if (n <= 0) return;                                   // uniform
@@ -1753,26 +1767,36 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
     const bool cok = c < Dv;
     const int g = h / (H / G);
     const int p0 = pos[(long)b * S];
+    const int tbeg = MODE == 0 ? 0 : min(n, sgi * seglen);
+    const int tend = MODE == 0 ? n : min(n, tbeg + seglen);
     float* sp = state + (((long)slot * H + h) * Dv + (cok ? c : 0)) * (long)D;
+    float* wp = MODE == 0 ? nullptr
+        : ws + ((((long)b * nseg + sgi) * H + h) * Dv + (cok ? c : 0)) * (long)D;
     float st[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int d = part + 16 * r;
-        st[r] = (cok && d < D && p0 > 0) ? sp[d] : 0.f;
+        float s0 = 0.f;
+        if (cok && d < D) {
+            if (MODE == 0) s0 = p0 > 0 ? sp[d] : 0.f;
+            else if (MODE == 2) s0 = wp[d];
+        }
+        st[r] = s0;
     }
     const float skp = skip ? skip[h] : 0.f;
-    for (int t0 = 0; t0 < n; t0 += DS_TC) {
-        const int cnt = min(DS_TC, n - t0);
+    float aprod = 1.f;
+    for (int t0 = tbeg; t0 < tend; t0 += DS_TC) {
+        const int cnt = min(DS_TC, tend - t0);
         __syncthreads();                                  // the previous chunk is consumed
         for (int idx = tid; idx < DS_TC * DP; idx += 256) {
             const int tt = idx / DP, d = idx % DP;
             float qv = 0.f, kv = 0.f;
             if (tt < cnt && d < D) {
                 const long tok = (long)b * S + t0 + tt;
-                qv = ldf<T>(q + tok * qs + (long)g * D + d);
+                if (MODE != 1) qv = ldf<T>(q + tok * qs + (long)g * D + d);
                 kv = ldf<T>(k + tok * ks + (long)g * D + d) * k_scale;
             }
-            sq[tt][d] = qv;
+            if (MODE != 1) sq[tt][d] = qv;
             sk[tt][d] = kv;
         }
         {
@@ -1797,26 +1821,58 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
         for (int tt = 0; tt < cnt; ++tt) {
             const float a = sa[tt], xv = sv[tt][cl];
             const float wv = sw[tt] * xv;
-            float acc = 0.f;
+            if (MODE == 1) {
+                aprod *= a;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int d = part + 16 * r;
-                st[r] = a * st[r] + sk[tt][d] * wv;
-                acc += st[r] * sq[tt][d];
+                for (int r = 0; r < R; ++r) st[r] = a * st[r] + sk[tt][part + 16 * r] * wv;
+            } else {
+                float acc = 0.f;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int d = part + 16 * r;
+                    st[r] = a * st[r] + sk[tt][d] * wv;
+                    acc += st[r] * sq[tt][d];
+                }
+                acc += __shfl_xor(acc, 8, WAVE);
+                acc += __shfl_xor(acc, 4, WAVE);
+                acc += __shfl_xor(acc, 2, WAVE);
+                acc += __shfl_xor(acc, 1, WAVE);
+                if (part == 0 && cok)
+                    out[(((long)b * S + t0 + tt) * H + h) * (long)Dv + c] = acc + skp * xv;
             }
-            acc += __shfl_xor(acc, 8, WAVE);
-            acc += __shfl_xor(acc, 4, WAVE);
-            acc += __shfl_xor(acc, 2, WAVE);
-            acc += __shfl_xor(acc, 1, WAVE);
-            if (part == 0 && cok)
-                out[(((long)b * S + t0 + tt) * H + h) * (long)Dv + c] = acc + skp * xv;
         }
     }
-    if (cok) {
+    if (MODE == 1 && c0 == 0 && tid == 0) wdec[((long)b * nseg + sgi) * H + h] = aprod;
+    float* dst = MODE == 1 ? wp : ((MODE == 0 || sgi == nseg - 1) ? sp : nullptr);
+    if (cok && dst) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int d = part + 16 * r;
-            if (d < D) sp[d] = st[r];
+            if (d < D) dst[d] = st[r];
+        }
+    }
+}
+
+// start states of the segments, in place over their end states (see above)
+__global__ void decay_scan_link_kernel(float* __restrict__ ws, const float* __restrict__ wdec,
+                                       const float* __restrict__ state,
+                                       const int* __restrict__ pos, const int* __restrict__ seq,
+                                       const int* __restrict__ nvalid, int B, int S, int H,
+                                       long per_head, int nseg) {
+    const long total = (long)B * H * per_head;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long e = i % per_head;
+        const int h = (i / per_head) % H;
+        const int b = i / (per_head * H);
+        const int slot = seq[b];
+        if (slot < 0 || nvalid[b] <= 0) continue;
+        float s = pos[(long)b * S] > 0 ? state[((long)slot * H + h) * per_head + e] : 0.f;
+        for (int c = 0; c < nseg; ++c) {
+            float* p = ws + (((long)b * nseg + c) * H + h) * per_head + e;
+            const float end = *p;
+            *p = s;
+            s = wdec[((long)b * nseg + c) * H + h] * s + end;
         }
     }
 }
@@ -2413,21 +2469,37 @@ int nx_decay_scan(const void* q, long qs, const void* k, long ks, const void* v,
                   int in_bf16, const void* dt, long dts, int dt_bf16, const float* dt_bias,
                   const float* a_log, const float* head_decay, float k_scale, const float* skip,
                   float* state, const int* pos, const int* seq, const int* nvalid, float* out,
-                  int B, int S, int H, int G, int D, int Dv, hipStream_t st) {
+                  int B, int S, int H, int G, int D, int Dv, float* ws, float* wdec, int nseg,
+                  int seglen, hipStream_t st) {
     if ((long)B * S <= 0) return 0;
     if (D <= 0 || Dv <= 0 || G <= 0 || H % G != 0 || D > 256) return -1;
     if ((dt == nullptr) == (head_decay == nullptr)) return -2;
     if (dt && (!dt_bias || !a_log)) return -2;
     if (H > 65535 || B > 65535) return -3;
-    dim3 grid((Dv + 15) / 16, H, B), block(256);
-#define DSK(T, TD, RV) decay_scan_kernel<T, TD, RV><<<grid, block, 0, st>>>( \
+    if (nseg < 1 || (nseg > 1 && (!ws || !wdec || seglen <= 0 || (long)nseg * seglen < S)))
+        return -4;
+    const int cb = (Dv + 15) / 16;
+    dim3 grid(cb * nseg, H, B), block(256);
+#define DSK(T, TD, RV, MD) decay_scan_kernel<T, TD, RV, MD><<<grid, block, 0, st>>>( \
         (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, (const TD*)dt, dts, dt_bias, a_log, \
-        head_decay, k_scale, skip, state, pos, seq, nvalid, out, S, H, G, D, Dv)
-#define DSR(T, TD) do { if (D <= 16) DSK(T, TD, 1); else if (D <= 32) DSK(T, TD, 2); \
-        else if (D <= 64) DSK(T, TD, 4); else if (D <= 128) DSK(T, TD, 8); \
-        else DSK(T, TD, 16); } while (0)
-    if (in_bf16) { if (dt_bf16) DSR(bf16, bf16); else DSR(bf16, float); }
-    else { if (dt_bf16) DSR(float, bf16); else DSR(float, float); }
+        head_decay, k_scale, skip, state, pos, seq, nvalid, out, S, H, G, D, Dv, ws, wdec, nseg, \
+        seglen)
+#define DSR(T, TD, MD) do { if (D <= 16) DSK(T, TD, 1, MD); else if (D <= 32) DSK(T, TD, 2, MD); \
+        else if (D <= 64) DSK(T, TD, 4, MD); else if (D <= 128) DSK(T, TD, 8, MD); \
+        else DSK(T, TD, 16, MD); } while (0)
+#define DST(MD) do { \
+        if (in_bf16) { if (dt_bf16) DSR(bf16, bf16, MD); else DSR(bf16, float, MD); } \
+        else { if (dt_bf16) DSR(float, bf16, MD); else DSR(float, float, MD); } } while (0)
+    if (nseg == 1) {
+        DST(0);
+    } else {
+        DST(1);
+        const long per_head = (long)Dv * D;
+        decay_scan_link_kernel<<<grid_for((long)B * H * per_head, 256), 256, 0, st>>>(
+            ws, wdec, state, pos, seq, nvalid, B, S, H, per_head, nseg);
+        DST(2);
+    }
+#undef DST
 #undef DSR
 #undef DSK
     return (int)hipGetLastError();

@@ -535,6 +535,19 @@ def decay_scan(q, k, v, state, step: StepLayout, dim: int, vdim: int, dt=None,
         assert state.is_contiguous() and tuple(state.shape[1:]) == (H, vdim, dim)
         assert H % G == 0 and q.shape[-1] == G * dim and k.shape[-1] == G * dim
         out = torch.empty(B, S, H * vdim, dtype=torch.float32, device=v.device)
+        # a long row with few (row, head, channel block) workgroups is cut into
+        # segments that scan side by side (two passes joined by a short serial
+        # link over the segments' end states)
+        groups = B * H * ((vdim + 15) // 16)
+        nseg, seglen, ws, wdec = 1, S, None, None
+        if S >= 256 and groups < 1024:
+            nseg = 1
+            while nseg * 2 <= min(S // 64, max(1, 2048 // groups)):
+                nseg *= 2
+            if nseg > 1:
+                seglen = ((S + nseg - 1) // nseg + 15) // 16 * 16
+                ws = torch.empty(B * nseg * H * vdim * dim, dtype=torch.float32, device=v.device)
+                wdec = torch.empty(B * nseg * H, dtype=torch.float32, device=v.device)
         _check(lib.nx_decay_scan(
             _p(q), ctypes.c_long(_rows_view(q)), _p(k), ctypes.c_long(_rows_view(k)),
             _p(v), ctypes.c_long(_rows_view(v)), _is_bf16(v),
@@ -545,7 +558,7 @@ def decay_scan(q, k, v, state, step: StepLayout, dim: int, vdim: int, dt=None,
             _p(None if head_decay is None else _f32(head_decay)),
             ctypes.c_float(k_scale), _p(None if skip is None else _f32(skip)),
             _p(state), _p(step.positions), _p(step.seq_ids), _p(step.nvalid), _p(out),
-            B, S, H, G, dim, vdim, _stream()), "decay_scan")
+            B, S, H, G, dim, vdim, _p(ws), _p(wdec), nseg, seglen, _stream()), "decay_scan")
         return out
     return ref.decay_scan(q, k, v, state, step.positions, step.seq_ids, dim, vdim,
                           dt=dt, dt_bias=dt_bias, a_log=a_log, head_decay=head_decay,

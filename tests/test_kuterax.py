@@ -942,3 +942,40 @@ def test_config_rejects_what_it_does_not_know():
     bad["loop"] = {"start": 2, "stop": 9, "times": 2}
     with pytest.raises(ValueError):
         KuteraxInferenceConfig(neuron_config=EngineConfig(tp_degree=1), **bad)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_state_space_long_prompt_then_decode(device):
+    """Long portions take the segmented scan on the GPU (segments side by
+    side, joined through their end states)."""
+    _ssd_alone(device, right_cfg(2, 20, 12, 1, 4, 2), 340, [300, 2, 37, 1], tol=1e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_decay_scan_unequal_long_rows(device):
+    """Rows of unequal length in one step, one continuing from a carried
+    state, one starting, one pad row: against the reference op on the CPU."""
+    from neuronx_distributed_inference_amd.ops import ref
+
+    torch.manual_seed(21)
+    B, S, H, G, D, Dv = 3, 330, 4, 2, 24, 20
+    q, k = torch.randn(B, S, G * D) * 0.3, torch.randn(B, S, G * D) * 0.3
+    v = torch.randn(B, S, H * Dv)
+    dt = torch.randn(B, S, H)
+    dt_bias, a_log, skip = torch.randn(H), torch.rand(H) - 1.0, torch.randn(H)
+    pos = torch.full((B, S), -1, dtype=torch.long)
+    pos[0, :330] = torch.arange(5, 335)          # continues
+    pos[1, :77] = torch.arange(0, 77)            # starts, short
+    state0 = torch.randn(4, H, Dv, D)
+    st_ref = state0.clone()
+    want = ref.decay_scan(q, k, v, st_ref, pos, torch.tensor([2, 0, -1]), D, Dv, dt=dt,
+                          dt_bias=dt_bias, a_log=a_log, skip=skip)
+    st_dev = state0.clone().to(device)
+    step = step_for(pos, [2, 0, -1], device)
+    got = seqmix.decay_scan(q.to(device), k.to(device), v.to(device), st_dev, step, D, Dv,
+                            dt=dt.to(device), dt_bias=dt_bias.to(device),
+                            a_log=a_log.to(device), skip=skip.to(device)).cpu()
+    close(got[0], want[0], 1e-4, rtol=1e-4)
+    close(got[1, :77], want[1, :77], 1e-4, rtol=1e-4)
+    close(st_dev.cpu()[[0, 2]], st_ref[[0, 2]], 1e-4, rtol=1e-4)
+    assert torch.equal(st_dev.cpu()[[1, 3]], state0[[1, 3]])      # untouched slots
