@@ -2041,6 +2041,23 @@ __global__ void relu2_scale_vec_kernel(const T* __restrict__ x, const float* __r
     }
 }
 
+// ------------------------------------------- embedding + learned position rows
+// stream[t, :] = float(emb[t, :]) + float(table[max(pos[t], 0), :])
+template <typename T>
+__global__ void embed_pos_kernel(const T* __restrict__ emb, const T* __restrict__ table,
+                                 const int* __restrict__ pos, float* __restrict__ out,
+                                 long ntok, int C, int rows_in_table) {
+    const long total = ntok * C;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C;
+        const int c = i % C;
+        int p = pos[t];
+        p = p < 0 ? 0 : (p >= rows_in_table ? rows_in_table - 1 : p);
+        out[i] = ldf<T>(emb + i) + ldf<T>(table + (long)p * C + c);
+    }
+}
+
 // ------------------------------------- residual sum of weighted, optionally normed terms
 // x[row] += sum_i f_i(y_i[row]) * w_i, f_i = RMS norm over the row or identity.
 // One workgroup per row; statistics fp32.
@@ -2056,14 +2073,15 @@ scaled_residual_kernel(float* __restrict__ x, const T* __restrict__ y0,
     const float* ws[3] = {w0, w1, w2};
     const int ns[3] = {n0, n1, n2};
     float inv[3] = {1.f, 1.f, 1.f};
+    float ss[3] = {0.f, 0.f, 0.f};
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
-        if (!ys[i] || !ns[i]) continue;                   // uniform
-        const T* yr = ys[i] + row * C;
-        float ss = 0.f;
-        for (int c = threadIdx.x; c < C; c += LN_THREADS) { const float v = ldf<T>(yr + c); ss += v * v; }
-        inv[i] = 1.f / sqrtf(block_sum(ss, red) / C + eps);
+        for (int i = 0; i < 3; ++i)
+            if (ys[i] && ns[i]) { const float v = ldf<T>(ys[i] + row * C + c); ss[i] += v * v; }
     }
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+        if (ys[i] && ns[i]) inv[i] = 1.f / sqrtf(block_sum(ss[i], red) / C + eps);   // uniform
     float* xr = x + row * C;
     for (int c = threadIdx.x; c < C; c += LN_THREADS) {
         float acc = 0.f;
@@ -2569,6 +2587,18 @@ int nx_scaled_residual(float* x, const void* y0, const float* w0, int n0, const 
         x, (const bf16*)y0, w0, n0, (const bf16*)y1, w1, n1, (const bf16*)y2, w2, n2, eps, C);
     else scaled_residual_kernel<float><<<grid, block, 0, st>>>(
         x, (const float*)y0, w0, n0, (const float*)y1, w1, n1, (const float*)y2, w2, n2, eps, C);
+    return (int)hipGetLastError();
+}
+
+int nx_embed_pos(const void* emb, const void* table, int is_bf16, const int* pos, float* out,
+                 long ntok, int C, int rows_in_table, hipStream_t st) {
+    if (ntok * C <= 0) return 0;
+    if (rows_in_table <= 0) return -1;
+    dim3 grid(grid_for(ntok * C, 256)), block(256);
+    if (is_bf16) embed_pos_kernel<bf16><<<grid, block, 0, st>>>(
+        (const bf16*)emb, (const bf16*)table, pos, out, ntok, C, rows_in_table);
+    else embed_pos_kernel<float><<<grid, block, 0, st>>>(
+        (const float*)emb, (const float*)table, pos, out, ntok, C, rows_in_table);
     return (int)hipGetLastError();
 }
 

@@ -657,5 +657,15 @@ def scaled_residual(x, terms, eps: float = 0.0):
 def embed_positions(h, pos_table, step: StepLayout):
     """Token embedding rows (B,S,W) plus a learned position row per token ->
     fp32 residual stream; pad tokens (position -1) take row 0."""
-    p = step.positions.long().clamp(min=0)
+    if h.is_cuda:
+        lib = _load()
+        h = h.contiguous()
+        assert pos_table.dtype == h.dtype and pos_table.is_contiguous()
+        W = h.shape[-1]
+        out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+        _check(lib.nx_embed_pos(_p(h), _p(pos_table), _is_bf16(h), _p(step.positions), _p(out),
+                                ctypes.c_long(h.numel() // W), W, pos_table.shape[0], _stream()),
+               "embed_positions")
+        return out
+    p = step.positions.long().clamp(min=0, max=pos_table.shape[0] - 1)
     return h.float() + pos_table[p].float()

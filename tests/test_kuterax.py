@@ -979,3 +979,14 @@ def test_decay_scan_unequal_long_rows(device):
     close(got[1, :77], want[1, :77], 1e-4, rtol=1e-4)
     close(st_dev.cpu()[[0, 2]], st_ref[[0, 2]], 1e-4, rtol=1e-4)
     assert torch.equal(st_dev.cpu()[[1, 3]], state0[[1, 3]])      # untouched slots
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_embed_positions_op(device):
+    torch.manual_seed(22)
+    emb = torch.randn(2, 4, 10)
+    table = torch.randn(7, 10)
+    pos = torch.tensor([[3, 4, 5, 6], [0, 1, -1, -1]])
+    got = seqmix.embed_positions(emb.to(device), table.to(device), step_for(pos, [0, 1], device))
+    want = emb.double() + table.double()[pos.clamp(min=0)]
+    close(got.cpu(), want, 1e-6)
