@@ -1708,17 +1708,16 @@ head_norm_rope_kernel(const TIn* __restrict__ x, long xt, long xh, TOut* __restr
         for (int c = lane; c < C; c += WAVE) row[c] = row[c] * inv * nw[c];
     }
     __builtin_amdgcn_wave_barrier();
-    for (int c = lane; c < C; c += WAVE) {
-        float o = row[c];
-        if (c < 2 * half) {
-            const int i = c < half ? c : c - half;
-            float sn, cs;
-            sincosf((float)p * inv_freq[i], &sn, &cs);
-            sn *= mscale; cs *= mscale;
-            o = c < half ? o * cs - row[c + half] * sn : o * cs + row[c - half] * sn;
-        }
-        stf<TOut>(op + c, o);
+    // a lane owns whole pairs: one sincos serves both channels
+    for (int i = lane; i < half; i += WAVE) {
+        float sn, cs;
+        sincosf((float)p * inv_freq[i], &sn, &cs);
+        sn *= mscale; cs *= mscale;
+        const float u = row[i], w2 = row[i + half];
+        stf<TOut>(op + i, u * cs - w2 * sn);
+        stf<TOut>(op + i + half, w2 * cs + u * sn);
     }
+    for (int c = 2 * half + lane; c < C; c += WAVE) stf<TOut>(op + c, row[c]);
 }
 
 // ----------------------------------------------- scalar-decay linear recurrence
@@ -2038,6 +2037,67 @@ __global__ void relu2_scale_vec_kernel(const T* __restrict__ x, const float* __r
 #pragma unroll
         for (int e = 0; e < 8; ++e) { const float r = fmaxf(v[e], 0.f); v[e] = r * r * gw; }
         store8<T>(out + t * C + c, v);
+    }
+}
+
+// 16-byte variant for rows of up to LN_THREADS * 8 * NV channels: every term is
+// read once and stays in registers between the statistics and the update
+template <typename T, int NV>
+__global__ void __launch_bounds__(LN_THREADS)
+scaled_residual_vec_kernel(float* __restrict__ x, const T* __restrict__ y0,
+                           const float* __restrict__ w0, int n0, const T* __restrict__ y1,
+                           const float* __restrict__ w1, int n1, const T* __restrict__ y2,
+                           const float* __restrict__ w2, int n2, float eps, int C) {
+    __shared__ float red[3][LN_THREADS / WAVE];
+    const long row = blockIdx.x;
+    const T* ys[3] = {y0, y1, y2};
+    const float* ws[3] = {w0, w1, w2};
+    const int ns[3] = {n0, n1, n2};
+    float val[3][NV][8];
+    float ss[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        if (!ys[i]) continue;                             // uniform
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int c = (j * LN_THREADS + threadIdx.x) * 8;
+            if (c < C) {
+                load8<T>(ys[i] + row * C + c, val[i][j]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss[i] += val[i][j][e] * val[i][j][e];
+            }
+        }
+    }
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const float t = wave_sum(ss[i]);
+        if (lane == 0) red[i][wv] = t;
+    }
+    __syncthreads();
+    float inv[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < LN_THREADS / WAVE; ++k) t += red[i][k];
+        inv[i] = (ys[i] && ns[i]) ? 1.f / sqrtf(t / C + eps) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int c = (j * LN_THREADS + threadIdx.x) * 8;
+        if (c >= C) continue;
+        float xv[8];
+        load8<float>(x + row * C + c, xv);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            if (!ys[i]) continue;
+            float wv8[8];
+            load8<float>(ws[i] + c, wv8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xv[e] += val[i][j][e] * inv[i] * wv8[e];
+        }
+        st8<float>(x + row * C + c, xv);
     }
 }
 
@@ -2583,6 +2643,19 @@ int nx_scaled_residual(float* x, const void* y0, const float* w0, int n0, const 
     if (rows <= 0) return 0;
     if (!y0 || !w0 || (y1 && !w1) || (y2 && !w2)) return -1;
     dim3 grid((unsigned)rows), block(LN_THREADS);
+    const bool al = (C % 8) == 0 && C <= LN_THREADS * 8 * 4 && ((uintptr_t)x % 16) == 0 &&
+        ((uintptr_t)y0 % 16) == 0 && ((uintptr_t)y1 % 16) == 0 && ((uintptr_t)y2 % 16) == 0 &&
+        ((uintptr_t)w0 % 16) == 0 && ((uintptr_t)w1 % 16) == 0 && ((uintptr_t)w2 % 16) == 0;
+    if (al) {
+#define SRV(T, NVV) scaled_residual_vec_kernel<T, NVV><<<grid, block, 0, st>>>( \
+        x, (const T*)y0, w0, n0, (const T*)y1, w1, n1, (const T*)y2, w2, n2, eps, C)
+#define SRN(T) do { if (C <= LN_THREADS * 8) SRV(T, 1); else if (C <= LN_THREADS * 16) SRV(T, 2); \
+                    else SRV(T, 4); } while (0)
+        if (is_bf16) SRN(bf16); else SRN(float);
+#undef SRN
+#undef SRV
+        return (int)hipGetLastError();
+    }
     if (is_bf16) scaled_residual_kernel<bf16><<<grid, block, 0, st>>>(
         x, (const bf16*)y0, w0, n0, (const bf16*)y1, w1, n1, (const bf16*)y2, w2, n2, eps, C);
     else scaled_residual_kernel<float><<<grid, block, 0, st>>>(

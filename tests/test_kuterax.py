@@ -367,9 +367,9 @@ def test_relu2_scale_op(device, E, ff, rest):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_scaled_residual_op(device):
+@pytest.mark.parametrize("C", [40, 37, 2304])             # 16-byte / scalar / two vectors a thread
+def test_scaled_residual_op(device, C):
     torch.manual_seed(7)
-    C = 40
     x = torch.randn(2, 3, C)
     ys = [torch.randn(2, 3, C) * s for s in (3.0, 0.2, 1.0)]
     ws = [torch.randn(C) for _ in range(3)]
