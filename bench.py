@@ -175,7 +175,7 @@ def run_hybrid_bench(args):
             # layers; the feed-forward activates ff columns per token: four of
             # sixteen experts of ff/8 plus a shared expert of ff/2
             mlp = {"kind": "moe", "expert": {"ff": ff // 8}, "shared": {"ff": ff // 2},
-                   "router": {"experts": 16, "top": 4, "scale": 2.5,
+                   "router": {"experts": 16, "top": 4, "scale": 1.5,
                               "groups": {"count": 4, "keep": 2}}}
             par = {"type": "parallel", "mlp": mlp, "mixer": {
                 "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,

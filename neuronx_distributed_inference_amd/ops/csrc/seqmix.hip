@@ -1723,7 +1723,7 @@ head_norm_rope_kernel(const TIn* __restrict__ x, long xt, long xh, TOut* __restr
 // ----------------------------------------------- scalar-decay linear recurrence
 // S_t = a_t S_{t-1} + k_t (w_t v_t)^T, o_t = S_t^T q_t (+ skip_h v_t), one scalar
 // decay per head and token. Workgroup = (row, head, 16 value channels); the 16
-// lanes of a channel split its key rows (lane p owns rows p, p+16, ...), the
+// lanes of a channel split its key rows (lane p owns rows p*R .. p*R+R-1), the
 // state sits in registers for the whole step and is read/written once. Tokens
 // are staged through LDS in chunks of DS_TC (q, k, v, decay, step size), so
 // global loads are coalesced and the serial loop reads only LDS.
@@ -1753,8 +1753,8 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
                   int D, int Dv, float* __restrict__ ws, float* __restrict__ wdec, int nseg,
                   int seglen) {
     constexpr int DP = 16 * R;
-    __shared__ float sq[MODE == 1 ? 1 : DS_TC][DP], sk[DS_TC][DP], sv[DS_TC][16], sa[DS_TC],
-        sw[DS_TC];
+    __shared__ __attribute__((aligned(16))) float sq[MODE == 1 ? 1 : DS_TC][DP], sk[DS_TC][DP];
+    __shared__ float sv[DS_TC][16], sa[DS_TC], sw[DS_TC];
     const int b = blockIdx.z, h = blockIdx.y;
     const int sgi = MODE == 0 ? 0 : blockIdx.x % nseg;
     const int c0 = (MODE == 0 ? blockIdx.x : blockIdx.x / nseg) * 16;
@@ -1774,7 +1774,7 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
     float st[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int d = part + 16 * r;
+        const int d = part * R + r;
         float s0 = 0.f;
         if (cok && d < D) {
             if (MODE == 0) s0 = p0 > 0 ? sp[d] : 0.f;
@@ -1820,17 +1820,35 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
         for (int tt = 0; tt < cnt; ++tt) {
             const float a = sa[tt], xv = sv[tt][cl];
             const float wv = sw[tt] * xv;
+            // a lane's key rows are contiguous: 16-byte LDS reads
+            float kr[R], qr[R];
+            if constexpr (R % 4 == 0) {
+#pragma unroll
+                for (int r = 0; r < R; r += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(&sk[tt][part * R + r]);
+                    kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
+                    if (MODE != 1) {
+                        const float4 q4 = *reinterpret_cast<const float4*>(&sq[tt][part * R + r]);
+                        qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    kr[r] = sk[tt][part * R + r];
+                    if (MODE != 1) qr[r] = sq[tt][part * R + r];
+                }
+            }
             if (MODE == 1) {
                 aprod *= a;
 #pragma unroll
-                for (int r = 0; r < R; ++r) st[r] = a * st[r] + sk[tt][part + 16 * r] * wv;
+                for (int r = 0; r < R; ++r) st[r] = a * st[r] + kr[r] * wv;
             } else {
                 float acc = 0.f;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    const int d = part + 16 * r;
-                    st[r] = a * st[r] + sk[tt][d] * wv;
-                    acc += st[r] * sq[tt][d];
+                    st[r] = a * st[r] + kr[r] * wv;
+                    acc += st[r] * qr[r];
                 }
                 acc += __shfl_xor(acc, 8, WAVE);
                 acc += __shfl_xor(acc, 4, WAVE);
@@ -1846,7 +1864,7 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
     if (cok && dst) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int d = part + 16 * r;
+            const int d = part * R + r;
             if (d < D) dst[d] = st[r];
         }
     }
