@@ -1772,15 +1772,25 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
     float* wp = MODE == 0 ? nullptr
         : ws + ((((long)b * nseg + sgi) * H + h) * Dv + (cok ? c : 0)) * (long)D;
     float st[R];
+    const float* src = MODE == 0 ? (p0 > 0 ? sp : nullptr) : (MODE == 2 ? wp : nullptr);
+    // a lane's rows are contiguous in memory too: 16-byte accesses when the
+    // row length allows (every state row then starts on a 16-byte boundary)
+    const bool v4 = (R % 4 == 0) && (D % 4 == 0);
+    if (v4) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int d = part * R + r;
-        float s0 = 0.f;
-        if (cok && d < D) {
-            if (MODE == 0) s0 = p0 > 0 ? sp[d] : 0.f;
-            else if (MODE == 2) s0 = wp[d];
+        for (int r = 0; r < R; r += 4) {
+            const int d = part * R + r;
+            float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (cok && src && d < D) s4 = *reinterpret_cast<const float4*>(src + d);
+            st[r] = s4.x; st[r + 1 < R ? r + 1 : r] = s4.y;
+            st[r + 2 < R ? r + 2 : r] = s4.z; st[r + 3 < R ? r + 3 : r] = s4.w;
         }
-        st[r] = s0;
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int d = part * R + r;
+            st[r] = (cok && src && d < D) ? src[d] : 0.f;
+        }
     }
     const float skp = skip ? skip[h] : 0.f;
     float aprod = 1.f;
@@ -1862,10 +1872,21 @@ decay_scan_kernel(const T* __restrict__ q, long qs, const T* __restrict__ k, lon
     if (MODE == 1 && c0 == 0 && tid == 0) wdec[((long)b * nseg + sgi) * H + h] = aprod;
     float* dst = MODE == 1 ? wp : ((MODE == 0 || sgi == nseg - 1) ? sp : nullptr);
     if (cok && dst) {
+        if (v4) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int d = part * R + r;
-            if (d < D) dst[d] = st[r];
+            for (int r = 0; r < R; r += 4) {
+                const int d = part * R + r;
+                if (d < D)
+                    *reinterpret_cast<float4*>(dst + d) = make_float4(
+                        st[r], st[r + 1 < R ? r + 1 : r], st[r + 2 < R ? r + 2 : r],
+                        st[r + 3 < R ? r + 3 : r]);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int d = part * R + r;
+                if (d < D) dst[d] = st[r];
+            }
         }
     }
 }
@@ -2572,6 +2593,8 @@ int nx_decay_scan(const void* q, long qs, const void* k, long ks, const void* v,
     if ((dt == nullptr) == (head_decay == nullptr)) return -2;
     if (dt && (!dt_bias || !a_log)) return -2;
     if (H > 65535 || B > 65535) return -3;
+    // the kernel reads state rows 16 bytes at a time when dim % 4 == 0
+    if (((uintptr_t)state % 16) != 0 || ((uintptr_t)ws % 16) != 0) return -5;
     if (nseg < 1 || (nseg > 1 && (!ws || !wdec || seglen <= 0 || (long)nseg * seglen < S)))
         return -4;
     const int cb = (Dv + 15) / 16;
