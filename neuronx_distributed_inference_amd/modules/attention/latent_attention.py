@@ -1,12 +1,16 @@
-"""Latent (low-rank KV) attention with a softmax sink.
+"""Latent (low-rank KV) attention with an optional softmax sink, sliding
+window and output gate.
 
 Each token stores only a normed latent ``c`` (``kv_rank`` channels) and one
 rotated key part shared by all heads (``rot_dim`` channels). Per head the
 unrotated key is ``W_uk c`` and the value ``W_uv c``; the score is
 ``(q_plain . k_plain + q_rot . k_rot) * scale``. Rotary positions use the
 interleaved pair layout on the first ``rot_dims`` channels of the rotated
-part. The softmax denominator carries one extra term ``exp(sink_h)`` per
-head: a key without a value, unscaled.
+part. With ``sink`` the softmax denominator carries one extra term
+``exp(sink_h)`` per head: a key without a value, unscaled. With ``window``
+query ``i`` sees keys ``i - window < j <= i`` only. A ``gate`` handed to
+the call multiplies the concatenated heads by ``sigmoid(gate)`` element by
+element.
 
 Steps that continue a sequence (decoded tokens, later prompt portions, mixed
 batches) are computed in the *absorbed* form, which never expands the cache:
@@ -29,6 +33,8 @@ down-projection) are the caller's.
 
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 import torch.nn as nn
 
@@ -40,7 +46,7 @@ from neuronx_distributed_inference_amd.ops import seqmix
 class LatentSinkAttention(nn.Module):
     def __init__(self, num_heads: int, dim: int, rot_dim: int, v_dim: int, kv_rank: int,
                  scale: float, eps: float, rope_base: float, rot_dims: int,
-                 dtype: torch.dtype, sink: bool = True):
+                 dtype: torch.dtype, sink: bool = True, window: Optional[int] = None):
         super().__init__()
         assert rot_dims <= rot_dim and rot_dims % 2 == 0
         self.num_heads = num_heads
@@ -49,6 +55,7 @@ class LatentSinkAttention(nn.Module):
         self.v_dim = v_dim
         self.kv_rank = kv_rank
         self.scale = float(scale)
+        self.window = None if window is None else int(window)
         self.row = kv_rank + rot_dim                      # one cache row
         self.latent_norm = StreamRMSNorm(kv_rank, eps=eps, one_plus=False)
         self.register_buffer("inv_freq", interleaved_inv_freq(rope_base, rot_dims),
@@ -69,9 +76,10 @@ class LatentSinkAttention(nn.Module):
 
     @torch.no_grad()           # inference only: the batched products write into views
     def forward(self, q: torch.Tensor, dkv: torch.Tensor, kv_mgr, cache_idx: int,
-                step: seqmix.StepLayout) -> torch.Tensor:
-        """q (B,S,H*(dim+rot_dim)), dkv (B,S,kv_rank+rot_dim): column slices
-        of a fused projection are fine. Returns (B,S,H*v_dim)."""
+                step: seqmix.StepLayout, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q (B,S,H*(dim+rot_dim)), dkv (B,S,kv_rank+rot_dim), gate
+        (B,S,H*v_dim) or None: column slices of a fused projection are fine.
+        Returns (B,S,H*v_dim)."""
         B, S = q.shape[0], q.shape[1]
         H, D, R, C = self.num_heads, self.dim, self.rot_dim, self.kv_rank
         T = B * S
@@ -86,7 +94,7 @@ class LatentSinkAttention(nn.Module):
                               kv_mgr.slot_mapping, step)
         q4 = q.unflatten(-1, (H, D + R))
         if getattr(step, "fresh", False):
-            return self._expanded(q4, row, step)
+            return self._expanded(q4, row, step, gate)
         # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
         qa = torch.empty(B, S, H, self.row, dtype=dt, device=q.device)
         torch.bmm(q4[..., :D].flatten(0, 1).transpose(0, 1), self.uk,
@@ -95,13 +103,15 @@ class LatentSinkAttention(nn.Module):
         k_cache = kc.data
         lat = seqmix.paged_attention(
             qa.view(B, S, H * self.row), k_cache, k_cache[..., :C], step, kv_mgr.block_table,
-            self.scale, H, sink=self.sink, out_dtype=dt)              # (B,S,H*C)
+            self.scale, H, window=self.window, sink=self.sink, out_dtype=dt)   # (B,S,H*C)
         out = torch.empty(B, S, H * self.v_dim, dtype=dt, device=q.device)
         torch.bmm(lat.view(T, H, C).transpose(0, 1), self.uv.transpose(1, 2),
                   out=out.view(T, H, self.v_dim).transpose(0, 1))
+        if gate is not None:
+            seqmix.sigmoid_gate_(out, gate)
         return out
 
-    def _expanded(self, q4: torch.Tensor, row: torch.Tensor, step) -> torch.Tensor:
+    def _expanded(self, q4: torch.Tensor, row: torch.Tensor, step, gate=None) -> torch.Tensor:
         """Whole prompts: per-head keys [W_uk c | k_rot] and values W_uv c of
         this step's tokens, attended in place: the (B, S) token grid is
         addressed as B pages of S tokens."""
@@ -118,4 +128,4 @@ class LatentSinkAttention(nn.Module):
         pages = torch.arange(B, device=q4.device, dtype=torch.int32).view(B, 1)
         return seqmix.paged_attention(
             qx.view(B, S, H * (D + R)), kx, vx, step, pages, self.scale, H,
-            sink=self.sink, out_dtype=dt)
+            window=self.window, sink=self.sink, gate=gate, out_dtype=dt)

@@ -93,3 +93,23 @@ class GatedMLP(nn.Module):
         g = self.gate_proj(x, sequence_parallel=sp)
         u = self.up_proj(x, sequence_parallel=sp)
         return self.down_proj(self.act_mul(g, u), sequence_parallel=sp)
+
+
+class SquaredReluMLP(nn.Module):
+    """Two-matrix feed-forward ``W_down(relu(W_up x)^2)``; the activation is
+    one kernel between the two GEMMs."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, tp_degree: int,
+                 dtype: torch.dtype, group=None):
+        super().__init__()
+        self.up_proj = ColumnParallelLinear(hidden_size, intermediate_size, dtype=dtype,
+                                            tp_degree=tp_degree, group=group)
+        self.down_proj = RowParallelLinear(intermediate_size, hidden_size, dtype=dtype,
+                                           tp_degree=tp_degree, group=group)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        hid = self.up_proj(x)
+        act = seqmix.relu2_scale(hid.reshape(-1, hid.shape[-1]), None, hid.shape[-1], 1)
+        return self.down_proj(act.view(hid.shape))

@@ -403,11 +403,13 @@ class GroupLimitedRouter(nn.Module):
     softmax scores over ALL experts times ``scale`` (renormalised over the
     chosen ones first when ``normalize``). Logits, softmax and selection are
     fp32. ``extra_gates`` further rows of the weight are per-token sigmoid
-    gates computed by the same fp32 product (a shared expert's gate)."""
+    gates computed by the same fp32 product (a shared expert's gate). With
+    ``correction`` a stored per-expert offset is added to the scores for the
+    choice only; the weights stay the uncorrected scores."""
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, n_groups: int = 1,
                  keep_groups: int = 1, scale: float = 1.0, normalize: bool = False,
-                 extra_gates: int = 0):
+                 extra_gates: int = 0, correction: bool = False):
         super().__init__()
         assert num_experts % max(n_groups, 1) == 0 and top_k <= num_experts
         self.num_experts = num_experts
@@ -420,6 +422,8 @@ class GroupLimitedRouter(nn.Module):
         self.normalize = bool(normalize)
         self.weight = nn.Parameter(
             torch.empty(num_experts + extra_gates, hidden_size, dtype=torch.float32))
+        self.correction = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32),
+                                       requires_grad=False) if correction else None
 
     def forward(self, x: torch.Tensor):
         """x (T, hidden) -> (dense (T, E + extra) fp32, idx (T, top_k) int32,
@@ -428,7 +432,8 @@ class GroupLimitedRouter(nn.Module):
 
         logits = F.linear(x.float(), self.weight)
         return seqmix.group_limited_router(logits, self.num_experts, self.top_k, self.n_groups,
-                                           self.keep_groups, self.scale, self.normalize)
+                                           self.keep_groups, self.scale, self.normalize,
+                                           correction=self.correction)
 
 
 class FusedUngatedExperts(nn.Module):
@@ -495,3 +500,90 @@ class GroupRoutedFeedForward(nn.Module):
         flat = h.reshape(-1, shape[-1])
         dense, _, _ = self.router(flat)
         return self.experts(flat, dense).view(shape)
+
+
+class FusedGatedExperts(nn.Module):
+    """Three-matrix experts ``W_down(g * sigmoid(alpha g) * (u + 1))`` with
+    ``g = min(W_gate x, limit)`` and ``u = clamp(W_up x, +-limit)``, stacked
+    so that ALL experts and an optional always-on shared expert (own size
+    and clamp) are two GEMMs: ``gate_up`` holds the gate rows of every
+    expert, then of the shared one, then the up rows in the same order;
+    ``down`` (hidden, E*ff + shared_ff) side by side. The routing weight
+    (zero for an unchosen expert, one for the shared expert) multiplies the
+    activation before the second product, whose fp32 accumulator carries the
+    sum over experts. Dense over the experts for the same reasons as
+    :class:`FusedUngatedExperts`: no data-dependent shapes, no host
+    synchronisation, a token's result independent of its batch."""
+
+    def __init__(self, num_experts: int, hidden_size: int, expert_ff: int, limit: float,
+                 dtype: torch.dtype, shared_ff: int = 0, shared_limit: float = 0.0,
+                 alpha: float = 1.702, tp_degree: int = 1):
+        super().__init__()
+        from neuronx_distributed_inference_amd.parallel.layers import (
+            ColumnParallelLinear,
+            RowParallelLinear,
+        )
+
+        assert tp_degree == 1
+        self.num_experts = num_experts
+        self.expert_ff = expert_ff
+        self.shared_ff = shared_ff
+        self.limit = float(limit)
+        self.shared_limit = float(shared_limit)
+        self.alpha = float(alpha)
+        inner = num_experts * expert_ff + shared_ff
+        self.gate_up = ColumnParallelLinear(hidden_size, 2 * inner, dtype=dtype, tp_degree=1)
+        self.down = RowParallelLinear(inner, hidden_size, dtype=dtype, tp_degree=1)
+
+    @staticmethod
+    def stack_gate_up(gates, ups, shared_gate=None, shared_up=None):
+        """[(ff, hidden)] * E gate and up matrices (+ the shared expert's)
+        -> fused (2 * (E*ff + shared_ff), hidden) weight."""
+        sg = [shared_gate] if shared_gate is not None else []
+        su = [shared_up] if shared_up is not None else []
+        return torch.cat(list(gates) + sg + list(ups) + su, dim=0)
+
+    stack_down = staticmethod(FusedUngatedExperts.stack_down)
+
+    def forward(self, x: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
+        """x (T, hidden); gates (T, >= E) fp32 dense routing weights."""
+        from neuronx_distributed_inference_amd.ops import seqmix
+
+        hid = self.gate_up(x)
+        return self.down(seqmix.clamped_glu_scale(
+            hid, gates, self.expert_ff, self.num_experts, self.limit, self.shared_limit,
+            self.alpha, out_dtype=hid.dtype))
+
+
+class IdentityRoutedFeedForward(nn.Module):
+    """Mixture of clamped gated experts behind a softmax router whose last
+    ``identity`` outputs are experts without tensors: chosen, they pass the
+    feed-forward's input through, times their weight. The softmax runs over
+    all ``num_experts + identity`` outputs; a stored correction shifts the
+    scores for the choice of the ``top_k`` only, the weights are the
+    uncorrected scores (not renormalised unless asked). An optional shared
+    expert runs for every token with weight one.
+
+    ``forward`` returns ``(y, coef)``: the experts' weighted sum, and the
+    (T, identity) fp32 weights of the pass-through experts (zero where not
+    chosen; None when the router has none) — the caller adds ``sum(coef) *
+    input``, which the post-norm residual kernel does in passing."""
+
+    def __init__(self, hidden_size: int, num_experts: int, identity: int, top_k: int,
+                 expert_ff: int, limit: float, dtype: torch.dtype, shared_ff: int = 0,
+                 shared_limit: float = 0.0, alpha: float = 1.702, scale: float = 1.0,
+                 normalize: bool = False, correction: bool = True):
+        super().__init__()
+        self.num_experts = num_experts
+        self.identity = identity
+        self.router = GroupLimitedRouter(hidden_size, num_experts + identity, top_k,
+                                         scale=scale, normalize=normalize, correction=correction)
+        self.experts = FusedGatedExperts(num_experts, hidden_size, expert_ff, limit, dtype,
+                                         shared_ff, shared_limit, alpha)
+
+    def forward(self, h: torch.Tensor):
+        shape = h.shape
+        flat = h.reshape(-1, shape[-1])
+        dense, _, _ = self.router(flat)
+        y = self.experts(flat, dense).view(shape)
+        return y, (dense[:, self.num_experts:] if self.identity else None)

@@ -85,7 +85,12 @@ class StreamRMSNorm(nn.Module):
         return seqmix.rms_norm(x, self.weight, self.eps, self.one_plus,
                                out_dtype=None if out is not None else self.out_dtype, out=out)
 
-    def add_into(self, stream: torch.Tensor, y: torch.Tensor, copy_dtype=None):
+    def add_into(self, stream: torch.Tensor, y: torch.Tensor, copy_dtype=None, extra=None,
+                 coef=None, next_weight=None):
+        """``stream += norm(y [+ sum(coef) * extra])``; hands back the new
+        stream in ``copy_dtype``, or its RMS norm under ``next_weight`` (the
+        pre-norm of the sublayer that follows) from the same pass."""
         from neuronx_distributed_inference_amd.ops import seqmix
 
-        return seqmix.add_rms_norm(stream, y, self.weight, self.eps, self.one_plus, copy_dtype)
+        return seqmix.add_rms_norm(stream, y, self.weight, self.eps, self.one_plus, copy_dtype,
+                                   extra=extra, coef=coef, next_weight=next_weight)

@@ -287,15 +287,17 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
 // Score of query i and key j, in order: q.k * scale * temp(i), temp(i) = 1 +
 // qt_coef * ln(floor((i+1)/qt_every) + 1) (qt_every = 0: none); minus
 // r1_h * log(1 + r2_h (i-j)) (r1 = null: none); cap * tanh(. / cap) (cap = 0:
-// none). Visible: j <= i and (i-j < window or j < keep); plain causal attention
-// passes window = INT_MAX. `sink` (per head, or null) adds exp(sink_h) to the
-// softmax denominator. K and V rows are addressed as slot*tok_stride +
+// none); a lone r1 (r2 = null) is a linear penalty r1_h * (i-j) instead.
+// Visible: j <= i and (i-j < window or j < keep); plain causal attention
+// passes window = INT_MAX. With cmask > 0 also only keys of the query's own block
+// of cmask positions (j >= floor(i/cmask)*cmask). `sink` (per head, or null)
+// adds exp(sink_h) to the softmax denominator. K and V rows are addressed as slot*tok_stride +
 // head*head_stride, so V may be a channel range of the K rows.
 // Workgroup (4 waves) = ATT_NQ query rows that share one KV head: HPW query
 // heads of the group x QT consecutive tokens of a batch row, so every K/V
 // line fetched serves all of them. The union of the rows' visible keys is
-// [0, min(keep, lo)) + [lo, i_max], lo = max(0, i_min-window+1); each row
-// masks by its own position (j <= i and (i-j < window or j < keep)). Waves
+// [0, min(keep, lo)) + [lo, i_max], lo = the larger of max(0, i_min-window+1)
+// and i_min's block start; each row masks by its own position. Waves
 // take 64-key tiles round-robin: a lane owns one key for the scores (q rows
 // broadcast from LDS, fp32 accumulate, online softmax per row), then the
 // wave's P tile goes through LDS and a lane owns value channels for P.V.
@@ -317,7 +319,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                    int bsz, int S, float scale, int window, int keep, int HPW, int QT,
                    int chunks, int lpr, int pws, long ktok, long khead, long vtok, long vhead,
                    int kvec, const float* __restrict__ sink, float cap, float qt_coef,
-                   int qt_every, int ghead) {
+                   int qt_every, int ghead, int cmask) {
     // lpr > 0 (decode shape only): P.V with 8 value channels per lane and
     // 64/lpr keys per step, 16-byte V loads; pws = floats of LDS per wave
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -326,7 +328,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     float* ps = qs + ATT_NQ * DkP;                       // ATT_WAVES * 64 * ATT_NQ
     float* cs = ps;                                      // merge area reuses the P tiles
     constexpr int ATT_THREADS = ATT_WAVES * WAVE;
-    __shared__ int rpos[ATT_NQ_MAX];
+    __shared__ int rpos[ATT_NQ_MAX], rclo[ATT_NQ_MAX];
     __shared__ float ra1[ATT_NQ_MAX], ra2[ATT_NQ_MAX], rtemp[ATT_NQ_MAX], rsink[ATT_NQ_MAX];
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
@@ -341,9 +343,10 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
         int p = -1;
         if (tq < QT && t0 + tq < S && hh < rep) p = pos[(long)b * S + t0 + tq];
         rpos[tid] = p;
+        rclo[tid] = (cmask > 0 && p >= 0) ? (p / cmask) * cmask : 0;
         const int h = g * rep + (hh < rep ? hh : 0);
         ra1[tid] = r1 ? r1[h] : 0.f;
-        ra2[tid] = r1 ? r2[h] : 0.f;
+        ra2[tid] = r2 ? r2[h] : 0.f;
         rsink[tid] = sink ? sink[h] : -INFINITY;
         rtemp[tid] = (qt_every > 0 && p >= 0)
             ? 1.f + qt_coef * logf((float)((p + 1) / qt_every) + 1.f) : 1.f;
@@ -369,7 +372,7 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
     __syncthreads();
 
     const int* bt = btab + (long)b * max_blocks;
-    const int lo = max(0, i_min - window + 1);
+    const int lo = max(max(0, i_min - window + 1), cmask > 0 ? (i_min / cmask) * cmask : 0);
     const int nfirst = min(keep, lo);
     const int n = nfirst + (i_max - lo + 1);
     const int ntiles = (n + WAVE - 1) / WAVE;
@@ -431,14 +434,17 @@ window_attn_kernel(const T* __restrict__ q, long qstride, const T* __restrict__ 
                 const int i = rpos[r];
                 if (i < 0) continue;                     // uniform
                 const int dist = i - j;
-                const bool vis = kvalid && dist >= 0 && (dist < window || j < keep);
+                const bool vis = kvalid && dist >= 0 && (dist < window || j < keep) &&
+                                 j >= rclo[r];
                 float sv = -INFINITY;
                 if (vis) {
                     sv = sc[r];
-                    if (r1) {                            // uniform
+                    if (r1 && r2) {                      // uniform
                         const float x = ra2[r] * (float)dist;
                         const float lg = sizeof(T) == 4 ? log1pf(x) : __logf(1.f + x);
                         sv -= ra1[r] * lg;
+                    } else if (r1) {
+                        sv -= ra1[r] * (float)dist;
                     }
                     if (cap > 0.f) sv = cap * tanhf(sv / cap);
                 }
@@ -642,7 +648,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                        long gstride, bf16* __restrict__ out, int H, int G, int Dk, int Dv,
                        int bsz, int S, float scale, int window, int keep, int QT, long ktok,
                        long khead, long vtok, long vhead, const float* __restrict__ sink,
-                       float cap, float qt_coef, int qt_every, int nsplit, int ghead) {
+                       float cap, float qt_coef, int qt_every, int nsplit, int ghead,
+                       int cmask) {
     constexpr int KB = MA_KT / 16;           // 16-key score blocks per tile
     constexpr int KS = DKP + 8;              // K tile row stride (elements)
     constexpr int VS = MA_KT + 8;            // V^T tile row stride
@@ -661,7 +668,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         const int tq = tid / rep, hh = tid % rep;
         rpos[tid] = (tq < QT && t0 + tq < S) ? pos[(long)b * S + t0 + tq] : -1;
         ra1[tid] = r1 ? r1[g * rep + hh] : 0.f;
-        ra2[tid] = r1 ? r2[g * rep + hh] : 0.f;
+        ra2[tid] = r2 ? r2[g * rep + hh] : 0.f;
         rsink[tid] = sink ? sink[g * rep + hh] : -INFINITY;
     }
     __syncthreads();
@@ -674,6 +681,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
     // this lane's query row (B operand of S^T): row = 16*wv + lr
     const int myrow = wv * 16 + lr;
     const int my_i = rpos[myrow];
+    const int my_clo = (cmask > 0 && my_i >= 0) ? (my_i / cmask) * cmask : 0;
     const float a1 = ra1[myrow], a2 = ra2[myrow];
     const float qscale = (qt_every > 0 && my_i >= 0)
         ? scale * (1.f + qt_coef * logf((float)((my_i + 1) / qt_every) + 1.f)) : scale;
@@ -690,7 +698,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         }
     }
     const int* bt = btab + (long)b * max_blocks;
-    const int lo = max(0, i_min - window + 1);
+    const int lo = max(max(0, i_min - window + 1), cmask > 0 ? (i_min / cmask) * cmask : 0);
+    const int clo_max = cmask > 0 ? (i_max / cmask) * cmask : 0;   // block start of the last row
     const int nfirst = min(keep, lo);
     const int n = nfirst + (i_max - lo + 1);
     float m_run = -INFINITY, l_run = 0.f;
@@ -802,7 +811,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
         // a tile every row of the workgroup sees whole (all but the diagonal
         // tiles of a causal prompt) needs no per-score mask
         const bool whole = nfirst == 0 && base + MA_KT <= n && lo + base + MA_KT - 1 <= i_min &&
-                           i_max - (lo + base) < window;
+                           i_max - (lo + base) < window && lo + base >= clo_max;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -828,11 +837,12 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                 const int mm = base + kb * 16 + lg * 4 + r;
                 const int j = mm < nfirst ? mm : lo + (mm - nfirst);
                 const int dist = my_i - j;
-                const bool vis = mm < n && my_i >= 0 && dist >= 0 && (dist < window || j < keep);
+                const bool vis = mm < n && my_i >= 0 && dist >= 0 && (dist < window || j < keep) &&
+                                 j >= my_clo;
                 float x = -INFINITY;
                 if (vis) {
                     x = acc[r] * qscale;
-                    if (r1) x -= a1 * __logf(1.f + a2 * (float)dist);
+                    if (r1) x -= r2 ? a1 * __logf(1.f + a2 * (float)dist) : a1 * (float)dist;
                     if (cap > 0.f) x = cap * fast_tanh_(x / cap);
                 }
                 sv[kb][r] = x;
@@ -935,7 +945,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
 // All four waves compute the (cheap) scores of a 32-key tile; wave w owns value
 // channels [128w, 128w+128), so a workgroup covers 512 of them and the key row
 // is fetched from memory once: global -> registers (next tile prefetched) -> LDS
-// row-major, then V^T is cut out of that LDS tile. Causal, optional sink.
+// row-major, then V^T is cut out of that LDS tile. Causal, optionally inside a
+// sliding window or the token's block of positions; optional sink.
 // Grid: (tokens x key splits, head chunks of 16 x value splits of 512, batch
 // rows). With nks > 1 key splits a workgroup scans every nks-th run of tiles and
 // leaves an unnormalised partial (fp32 values, running max, sum) in `ws`;
@@ -950,7 +961,7 @@ latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* 
                           const int* __restrict__ btab, int max_blocks,
                           const float* __restrict__ sink, bf16* __restrict__ out, int H, int Dk,
                           int Dv, int bsz, int S, float scale, int nsplit, int nks,
-                          float* __restrict__ ws) {
+                          float* __restrict__ ws, int window, int cmask) {
     constexpr int KS = DKP + 8;
     constexpr int VS = LD_KT + 8;
     constexpr int VCH = 4 * LD_VW;
@@ -979,10 +990,12 @@ latent_decode_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* 
         }
     }
     const int* bt = btab + (long)b * max_blocks;
-    // this split's keys [k_lo, n): a contiguous run of 32-key tiles
-    const int tiles = (p + 1 + LD_KT - 1) / LD_KT, per = (tiles + nks - 1) / nks;
-    const int k_lo = ksp * per * LD_KT;
-    const int n = min(p + 1, (ksp + 1) * per * LD_KT);
+    // the token sees keys [first, p]; this split's keys [k_lo, n) are a
+    // contiguous run of 32-key tiles counted from `first`
+    const int first = max(max(0, p - window + 1), cmask > 0 ? (p / cmask) * cmask : 0);
+    const int tiles = (p + 1 - first + LD_KT - 1) / LD_KT, per = (tiles + nks - 1) / nks;
+    const int k_lo = first + ksp * per * LD_KT;
+    const int n = min(p + 1, first + (ksp + 1) * per * LD_KT);
     float m_run = -INFINITY, l_run = 0.f;
     f32x4_t o_acc[LD_VW / 16];
 #pragma unroll
@@ -1520,33 +1533,68 @@ rms_norm_vec_kernel(const TIn* __restrict__ x, long xs, const float* __restrict_
     }
 }
 
+// post-norm residual step: stream[row] += rms_norm(v[row]) * (w | 1 + w) in fp32,
+// v = y, or y + (sum of the row's `nc` coefficients) * extra (experts that pass
+// their input through). `copy` (optional) receives the updated row in the next
+// GEMM's input type, or, with `next_w`, the next sublayer's pre-norm
+// rms_norm(updated row) * next_w: the row's new statistics come from the same
+// pass that updates it.
 template <typename TY, typename TC>
 __global__ void __launch_bounds__(LN_THREADS)
 add_rms_norm_vec_kernel(float* __restrict__ stream, const TY* __restrict__ y,
                         const float* __restrict__ w, int one_plus, float eps,
-                        TC* __restrict__ copy, int C) {
+                        TC* __restrict__ copy, const TY* __restrict__ extra,
+                        const float* __restrict__ coef, long cs, int nc,
+                        const float* __restrict__ next_w, int C) {
     __shared__ float red[LN_THREADS / WAVE];
     const long row = blockIdx.x;
     const TY* yr = y + row * C;
+    const TY* er = extra ? extra + row * C : nullptr;
+    float cf = 0.f;
+    if (er) for (int k = 0; k < nc; ++k) cf += coef[row * cs + k];
     float s = 0.f;
     for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
         float v[8];
         load8<TY>(yr + c, v);
+        if (er) {
+            float ev[8];
+            load8<TY>(er + c, ev);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += cf * ev[e];
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) s += v[e] * v[e];
     }
     const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
     const float add = one_plus ? 1.f : 0.f;
     float* xr = stream + row * C;
+    float s2 = 0.f;
     for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
         float v[8], wv[8], xv[8];
         load8<TY>(yr + c, v);
+        if (er) {
+            float ev[8];
+            load8<TY>(er + c, ev);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += cf * ev[e];
+        }
         load8<float>(w + c, wv);
         load8<float>(xr + c, xv);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) xv[e] += v[e] * inv * (wv[e] + add);
+        for (int e = 0; e < 8; ++e) { xv[e] += v[e] * inv * (wv[e] + add); s2 += xv[e] * xv[e]; }
         store8<float>(xr + c, xv);
-        if (copy) store8<TC>(copy + row * C + c, xv);
+        if (copy && !next_w) store8<TC>(copy + row * C + c, xv);
+    }
+    if (!copy || !next_w) return;                        // uniform
+    __syncthreads();                                     // `red` is reused
+    const float inv2 = 1.f / sqrtf(block_sum(s2, red) / C + eps);
+    for (int c = threadIdx.x * 8; c < C; c += LN_THREADS * 8) {
+        float xv[8], wv[8];
+        load8<float>(xr + c, xv);                        // this thread's own stores
+        load8<float>(next_w + c, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[e] = xv[e] * inv2 * wv[e];
+        store8<TC>(copy + row * C + c, xv);
     }
 }
 
@@ -1566,26 +1614,41 @@ rms_norm_kernel(const TIn* __restrict__ x, long xs, const float* __restrict__ w,
         stf<TOut>(o + c, ldf<TIn>(xr + c) * inv * (w[c] + add));
 }
 
-// post-norm residual step: stream[row] += rms_norm(y[row]) * (w | 1 + w), fp32;
-// optionally also writes the updated row in the next GEMM's input type
+// scalar form of add_rms_norm_vec_kernel (any width and alignment)
 template <typename TY, typename TC>
 __global__ void __launch_bounds__(LN_THREADS)
 add_rms_norm_kernel(float* __restrict__ stream, const TY* __restrict__ y,
                     const float* __restrict__ w, int one_plus, float eps,
-                    TC* __restrict__ copy, int C) {
+                    TC* __restrict__ copy, const TY* __restrict__ extra,
+                    const float* __restrict__ coef, long cs, int nc,
+                    const float* __restrict__ next_w, int C) {
     __shared__ float red[LN_THREADS / WAVE];
     const long row = blockIdx.x;
     const TY* yr = y + row * C;
+    const TY* er = extra ? extra + row * C : nullptr;
+    float cf = 0.f;
+    if (er) for (int k = 0; k < nc; ++k) cf += coef[row * cs + k];
     float s = 0.f;
-    for (int c = threadIdx.x; c < C; c += LN_THREADS) { const float v = ldf<TY>(yr + c); s += v * v; }
+    for (int c = threadIdx.x; c < C; c += LN_THREADS) {
+        const float v = ldf<TY>(yr + c) + (er ? cf * ldf<TY>(er + c) : 0.f);
+        s += v * v;
+    }
     const float inv = 1.f / sqrtf(block_sum(s, red) / C + eps);
     const float add = one_plus ? 1.f : 0.f;
     float* xr = stream + row * C;
+    float s2 = 0.f;
     for (int c = threadIdx.x; c < C; c += LN_THREADS) {
-        const float v = xr[c] + ldf<TY>(yr + c) * inv * (w[c] + add);
+        const float yv = ldf<TY>(yr + c) + (er ? cf * ldf<TY>(er + c) : 0.f);
+        const float v = xr[c] + yv * inv * (w[c] + add);
         xr[c] = v;
-        if (copy) stf<TC>(copy + row * C + c, v);
+        s2 += v * v;
+        if (copy && !next_w) stf<TC>(copy + row * C + c, v);
     }
+    if (!copy || !next_w) return;                        // uniform
+    __syncthreads();
+    const float inv2 = 1.f / sqrtf(block_sum(s2, red) / C + eps);
+    for (int c = threadIdx.x; c < C; c += LN_THREADS)
+        stf<TC>(copy + row * C + c, xr[c] * inv2 * next_w[c]);
 }
 
 // ---------------------------------------------------------- rotary positions
@@ -1957,6 +2020,8 @@ __global__ void group_gated_norm_kernel(const float* __restrict__ y, const TG* _
 // (ties: lowest index). Writes the dense (T, E + extra) weight row (zeros at
 // unchosen experts, sigmoid gates in the extra columns), the chosen indices and
 // their weights = score * scale (renormalised over the chosen first if asked).
+// `corr` (E, or null) is added to the scores for the group ranking and the choice
+// only.
 // A row whose logits are not numbers (the garbage of a pad token) selects the
 // first experts with weight zero: every index stays in range.
 DEV void wave_argmax(float& v, int& i) {
@@ -1972,14 +2037,16 @@ DEV void wave_argmax(float& v, int& i) {
 __global__ void __launch_bounds__(RT_WAVES * WAVE)
 group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra, int top,
                     int ngroups, int keep, float scale, int normalize,
+                    const float* __restrict__ corr,
                     float* __restrict__ dense, int* __restrict__ idx, float* __restrict__ wts,
                     long T) {
-    extern __shared__ float rsm[];                        // per wave: E scores + ngroups
+    extern __shared__ float rsm[];                // per wave: E choice scores + ngroups + E scores
     const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
     const long t = (long)blockIdx.x * RT_WAVES + wv;
     if (t >= T) return;
-    float* cand = rsm + (long)wv * (E + ngroups);
+    float* cand = rsm + (long)wv * (2 * E + ngroups);
     float* gsc = cand + E;
+    float* sco = gsc + ngroups;                   // the uncorrected scores (the weights)
     const float* lp = logits + t * ls;
     float m = -INFINITY;
     for (int e = lane; e < E; e += WAVE) m = fmaxf(m, lp[e]);
@@ -1989,42 +2056,48 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
     sum = wave_sum(sum);
     const float rs = 1.f / sum;
     float* dp = dense + t * (long)(E + extra);
-    for (int e = lane; e < E; e += WAVE) { cand[e] *= rs; dp[e] = 0.f; }
+    for (int e = lane; e < E; e += WAVE) {
+        const float sc = cand[e] * rs;
+        sco[e] = sc;
+        cand[e] = corr ? sc + corr[e] : sc;       // the choice goes by the corrected score
+        dp[e] = 0.f;
+    }
     for (int x = lane; x < extra; x += WAVE) dp[E + x] = sigmoidf_(lp[E + x]);
     __builtin_amdgcn_wave_barrier();
     const int per = E / ngroups;
     if (ngroups > 1 && keep < ngroups) {
         for (int gi = lane; gi < ngroups; gi += WAVE) {
-            float gm = -1.f;
+            float gm = -INFINITY;
             for (int j = 0; j < per; ++j) gm = fmaxf(gm, cand[gi * per + j]);
             gsc[gi] = gm;
         }
         __builtin_amdgcn_wave_barrier();
         for (int r = 0; r < keep; ++r) {
-            float bv = -2.f; int bi = 0x7fffffff;
+            float bv = -INFINITY; int bi = 0x7fffffff;
             for (int gi = lane; gi < ngroups; gi += WAVE) {
                 const float x = gsc[gi];
-                if (x <= 1.5f && (x > bv)) { bv = x; bi = gi; }
+                if (x < INFINITY && (x > bv)) { bv = x; bi = gi; }
             }
             wave_argmax(bv, bi);
             if ((unsigned)bi >= (unsigned)ngroups) bi = r;   // a row of NaNs compares false everywhere
-            if (lane == 0) gsc[bi] = 2.f;                 // kept (scores are <= 1)
+            if (lane == 0) gsc[bi] = INFINITY;            // kept
             __builtin_amdgcn_wave_barrier();
         }
-        for (int e = lane; e < E; e += WAVE) if (gsc[e / per] != 2.f) cand[e] = -1.f;
+        for (int e = lane; e < E; e += WAVE) if (gsc[e / per] != INFINITY) cand[e] = -INFINITY;
         __builtin_amdgcn_wave_barrier();
     }
     float wsum = 0.f;
     float myw = 0.f; int myi = 0;                         // lane r keeps the r-th choice
     for (int r = 0; r < top; ++r) {
-        float bv = -2.f; int bi = 0x7fffffff;
+        float bv = -INFINITY; int bi = 0x7fffffff;
         for (int e = lane; e < E; e += WAVE) {
             const float x = cand[e];
             if (x > bv) { bv = x; bi = e; }
         }
         wave_argmax(bv, bi);
         if ((unsigned)bi >= (unsigned)E) { bi = r; bv = 0.f; }   // NaN row (a pad token): any valid index
-        if (lane == 0) cand[bi] = -3.f;
+        else bv = sco[bi];                                // the weight is the score itself
+        if (lane == 0) cand[bi] = -INFINITY;
         if (lane == (r & (WAVE - 1))) {
             // more than 64 choices: flush the previous one first
             if (r >= WAVE) { idx[t * top + r - WAVE] = myi; wts[t * top + r - WAVE] = myw; }
@@ -2044,7 +2117,7 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
 }
 
 // -------------------------------------------------- relu^2 times routing weight
-// out[t, c] = relu(x[t, c])^2 * gates[t, min(c / ff, E)]
+// out[t, c] = relu(x[t, c])^2 * gates[t, min(c / ff, E)] (gates = null: times one)
 template <typename T>
 __global__ void relu2_scale_kernel(const T* __restrict__ x, const float* __restrict__ gates,
                                    int gcols, int ff, int E, T* __restrict__ out, long rows,
@@ -2056,7 +2129,7 @@ __global__ void relu2_scale_kernel(const T* __restrict__ x, const float* __restr
         const int c = i % C;
         const int e = min(c / ff, E);
         const float v = fmaxf(ldf<T>(x + i), 0.f);
-        stf<T>(out + i, v * v * gates[t * gcols + e]);
+        stf<T>(out + i, v * v * (gates ? gates[t * gcols + e] : 1.f));
     }
 }
 
@@ -2070,12 +2143,97 @@ __global__ void relu2_scale_vec_kernel(const T* __restrict__ x, const float* __r
          i += (long)gridDim.x * blockDim.x) {
         const long t = i / C8;
         const int c = (i % C8) * 8;
-        const float gw = gates[t * gcols + min(c / ff, E)];
+        const float gw = gates ? gates[t * gcols + min(c / ff, E)] : 1.f;
         float v[8];
         load8<T>(x + t * C + c, v);
 #pragma unroll
         for (int e = 0; e < 8; ++e) { const float r = fmaxf(v[e], 0.f); v[e] = r * r * gw; }
         store8<T>(out + t * C + c, v);
+    }
+}
+
+// --------------------------------- clamped gated units of stacked experts
+// x (rows, 2C) = [gate | up] pre-activations of C = E*ff + shared columns.
+// out[t, c] = glu(gate, up; limit) * gates[t, c / ff] for c < E*ff (an expert's
+// columns, times the token's routing weight), glu(gate, up; shared_limit) for the
+// rest (an always-on shared expert); glu = g sigmoid(alpha g) (u + 1) on the
+// clamped pre-activations.
+template <typename T>
+__global__ void clamped_glu_scale_kernel(const T* __restrict__ x, const float* __restrict__ gates,
+                                         long gs, int ff, int E, float limit, float slimit,
+                                         float alpha, T* __restrict__ out, long rows, int C) {
+    const long total = rows * C;
+    const int ne = E * ff;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C;
+        const int c = i % C;
+        const bool own = c < ne;
+        const float gw = own ? gates[t * gs + c / ff] : 1.f;
+        float o = 0.f;
+        if (gw != 0.f)
+            o = clamped_glu_(ldf<T>(x + t * 2 * C + c), ldf<T>(x + t * 2 * C + C + c),
+                             own ? limit : slimit, alpha) * gw;
+        stf<T>(out + i, o);
+    }
+}
+
+template <typename T>
+__global__ void clamped_glu_scale_vec_kernel(const T* __restrict__ x,
+                                             const float* __restrict__ gates, long gs, int ff,
+                                             int E, float limit, float slimit, float alpha,
+                                             T* __restrict__ out, long rows, int C) {
+    const int C8 = C / 8;
+    const long total = rows * C8;
+    const int ne = E * ff;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C8;
+        const int c = (i % C8) * 8;                      // ff % 8 == 0: one owner per 8 columns
+        const bool own = c < ne;
+        const float gw = own ? gates[t * gs + c / ff] : 1.f;
+        float o[8];
+        if (gw != 0.f) {                                 // an unchosen expert's columns are not read
+            float g[8], u[8];
+            load8<T>(x + t * 2 * C + c, g);
+            load8<T>(x + t * 2 * C + C + c, u);
+            const float lim = own ? limit : slimit;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = clamped_glu_(g[e], u[e], lim, alpha) * gw;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = 0.f;
+        }
+        store8<T>(out + t * C + c, o);
+    }
+}
+
+// y[t, c] *= sigmoid(gate[t, c]); gate rows may be a column slice (row stride gs)
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, const T* __restrict__ gate, long gs,
+                                    long rows, int C, int vec) {
+    if (vec) {
+        const int C8 = C / 8;
+        const long total = rows * C8;
+        for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+             i += (long)gridDim.x * blockDim.x) {
+            const long t = i / C8;
+            const int c = (i % C8) * 8;
+            float v[8], g[8];
+            load8<T>(y + t * C + c, v);
+            load8<T>(gate + t * gs + c, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= sigmoidf_(g[e]);
+            store8<T>(y + t * C + c, v);
+        }
+        return;
+    }
+    const long total = rows * C;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)gridDim.x * blockDim.x) {
+        const long t = i / C;
+        const int c = i % C;
+        stf<T>(y + i, ldf<T>(y + i) * sigmoidf_(ldf<T>(gate + t * gs + c)));
     }
 }
 
@@ -2282,11 +2440,12 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
                   const float* sink, const void* gate, long gstride, void* out, int io_bf16,
                   int out_bf16, int B, int S, int H, int G, int Dk, int Dv, int bsz,
                   float scale, int window, int keep, float cap, float qt_coef, int qt_every,
-                  float* ws, int nks, int ghead, hipStream_t st) {
+                  float* ws, int nks, int ghead, int cmask, hipStream_t st) {
     if ((long)B * S <= 0) return 0;
     if (Dv > WAVE * 8 || H % G != 0 || Dk <= 0 || Dv <= 0) return -1;
     if (!io_bf16 && out_bf16) return -2;
-    if ((r1 == nullptr) != (r2 == nullptr)) return -4;
+    if (r2 != nullptr && r1 == nullptr) return -4;
+    if (cmask < 0 || window < 1) return -7;
     const int esz = io_bf16 ? 2 : 4;
     const int vecn = 16 / esz;                            // elements per 16-byte load
     const bool k_al = (Dk % 8) == 0 && (ktok % vecn) == 0 && (khead % vecn) == 0 &&
@@ -2294,7 +2453,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
     const bool v_al = (Dv % 8) == 0 && (vtok % vecn) == 0 && (vhead % vecn) == 0 &&
                       ((uintptr_t)vc % 16) == 0;
     if (io_bf16 && out_bf16 && S == 1 && G == 1 && vc == kc && vtok == ktok && k_al && v_al &&
-        !r1 && !gate && cap <= 0.f && qt_every <= 0 && window == 0x7fffffff && H >= 8 &&
+        !r1 && !gate && cap <= 0.f && qt_every <= 0 && keep == 0 && H >= 8 &&
         Dk <= 640 && (qstride % 8) == 0 && ((uintptr_t)q % 16) == 0) {
         // latent caches, single-token steps: one workgroup per token reads each
         // key row once and covers 512 value channels
@@ -2313,7 +2472,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
             } \
             latent_decode_mfma_kernel<DKV><<<gl, bl, lsh, st>>>( \
                 (const bf16*)q, qstride, (const bf16*)kc, ktok, pos, seq, btab, max_blocks, sink, \
-                (bf16*)out, H, Dk, Dv, bsz, S, scale, nsplit, nks, ws); } while (0)
+                (bf16*)out, H, Dk, Dv, bsz, S, scale, nsplit, nks, ws, window, cmask); } while (0)
         if (dkp <= 128) LD(128);
         else if (dkp <= 256) LD(256);
         else if (dkp <= 384) LD(384);
@@ -2346,7 +2505,7 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
 #define MA(DKV, DVV, KTV) paged_attn_mfma_kernel<DKV, DVV, KTV, (KTV == 32)><<<gm, bm, 0, st>>>( \
         (const bf16*)q, qstride, (const bf16*)kc, (const bf16*)vc, pos, seq, btab, max_blocks, \
         r1, r2, (const bf16*)gate, gstride, (bf16*)out, H, G, Dk, Dv, bsz, S, scale, window, \
-        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit, ghead)
+        keep, QTm, ktok, khead, vtok, vhead, sink, cap, qt_coef, qt_every, nsplit, ghead, cmask)
 #define MAV(DKV) do { if (dvp == 32) MA(DKV, 32, 64); else if (dvp == 64) MA(DKV, 64, 64); \
                       else if (dvp == 96) MA(DKV, 96, 64); else MA(DKV, 128, 64); } while (0)
             if (wide) {
@@ -2400,7 +2559,8 @@ int nx_paged_attn(const void* q, long qstride, const void* kc, long ktok, long k
     window_attn_kernel<T, TO, MR, Q, W><<<grid, block, sh, st>>>( \
         (const T*)q, qstride, (const T*)kc, (const T*)vc, pos, seq, btab, max_blocks, r1, r2, \
         (const T*)gate, gstride, (TO*)out, H, G, Dk, Dv, bsz, S, scale, window, keep, HPW, QT, \
-        chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every, ghead)
+        chunks, lpr, pws, ktok, khead, vtok, vhead, kvec, sink, cap, qt_coef, qt_every, ghead, \
+        cmask)
 #define WAS(T, TO, MR) do { if (dec) { WA(T, TO, MR, 4, 16); } else { WA(T, TO, MR, 16, 4); } } while (0)
 #define WAM(T, TO) do { if (Dv <= 2 * WAVE) WAS(T, TO, 2); else if (Dv <= 4 * WAVE) WAS(T, TO, 4); \
                         else WAS(T, TO, 8); } while (0)
@@ -2510,22 +2670,22 @@ int nx_rms_norm(const void* x, long xs, int x_bf16, const float* w, int one_plus
 }
 
 int nx_add_rms_norm(float* stream, const void* y, int y_bf16, const float* w, int one_plus,
-                    float eps, void* copy_bf16, long rows, int C, hipStream_t st) {
+                    float eps, void* copy, int copy_bf16, const void* extra, const float* coef,
+                    long cs, int nc, const float* next_w, long rows, int C, hipStream_t st) {
     if (rows <= 0) return 0;
+    if ((extra == nullptr) != (coef == nullptr)) return -1;
     dim3 grid((unsigned)rows), block(LN_THREADS);
     const bool vec = (C % 8) == 0 && ((uintptr_t)stream % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
-                     ((uintptr_t)copy_bf16 % 16) == 0 && ((uintptr_t)w % 16) == 0;
-    if (vec) {
-        if (y_bf16) add_rms_norm_vec_kernel<bf16, bf16><<<grid, block, 0, st>>>(
-            stream, (const bf16*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
-        else add_rms_norm_vec_kernel<float, bf16><<<grid, block, 0, st>>>(
-            stream, (const float*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
-        return (int)hipGetLastError();
-    }
-    if (y_bf16) add_rms_norm_kernel<bf16, bf16><<<grid, block, 0, st>>>(
-        stream, (const bf16*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
-    else add_rms_norm_kernel<float, bf16><<<grid, block, 0, st>>>(
-        stream, (const float*)y, w, one_plus, eps, (bf16*)copy_bf16, C);
+                     ((uintptr_t)copy % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+                     ((uintptr_t)extra % 16) == 0 && ((uintptr_t)next_w % 16) == 0;
+#define ARN(K, TY, TC) K<TY, TC><<<grid, block, 0, st>>>(stream, (const TY*)y, w, one_plus, eps, \
+        (TC*)copy, (const TY*)extra, coef, cs, nc, next_w, C)
+#define ARN2(K) do { if (y_bf16 && copy_bf16) ARN(K, bf16, bf16); else if (y_bf16) ARN(K, bf16, float); \
+                     else if (copy_bf16) ARN(K, float, bf16); else ARN(K, float, float); } while (0)
+    if (vec) ARN2(add_rms_norm_vec_kernel);
+    else ARN2(add_rms_norm_kernel);
+#undef ARN2
+#undef ARN
     return (int)hipGetLastError();
 }
 
@@ -2642,23 +2802,23 @@ int nx_group_gated_norm(const float* y, const void* gate, long gs, int gate_bf16
 }
 
 int nx_group_router(const float* logits, long ls, int E, int extra, int top, int ngroups,
-                    int keep, float scale, int normalize, float* dense, int* idx, float* wts,
-                    long T, hipStream_t st) {
+                    int keep, float scale, int normalize, const float* corr, float* dense,
+                    int* idx, float* wts, long T, hipStream_t st) {
     if (T <= 0) return 0;
     if (E <= 0 || top <= 0 || top > E || top > WAVE || ngroups <= 0 || E % ngroups != 0 ||
         keep <= 0 || keep > ngroups || (long)top > (long)(E / ngroups) * keep) return -1;
-    const size_t sh = (size_t)RT_WAVES * (E + ngroups) * sizeof(float);
+    const size_t sh = (size_t)RT_WAVES * (2 * E + ngroups) * sizeof(float);
     if (sh > 60 * 1024) return -2;
     dim3 grid((unsigned)((T + RT_WAVES - 1) / RT_WAVES)), block(RT_WAVES * WAVE);
     group_router_kernel<<<grid, block, sh, st>>>(logits, ls, E, extra, top, ngroups, keep, scale,
-                                                 normalize, dense, idx, wts, T);
+                                                 normalize, corr, dense, idx, wts, T);
     return (int)hipGetLastError();
 }
 
 int nx_relu2_scale(const void* x, int is_bf16, const float* gates, int gcols, int ff, int E,
                    void* out, long rows, int C, hipStream_t st) {
     if (rows * C <= 0) return 0;
-    if (ff <= 0 || gcols < E || (C > E * ff && gcols < E + 1)) return -1;
+    if (ff <= 0 || (gates && (gcols < E || (C > E * ff && gcols < E + 1)))) return -1;
     const int esz = is_bf16 ? 2 : 4;
     const bool vec = (C % 8) == 0 && (ff % 8) == 0 && ((uintptr_t)x % 16) == 0 &&
                      ((uintptr_t)out % 16) == 0 && esz > 0;
@@ -2675,6 +2835,44 @@ int nx_relu2_scale(const void* x, int is_bf16, const float* gates, int gcols, in
         else relu2_scale_kernel<float><<<grid, block, 0, st>>>(
             (const float*)x, gates, gcols, ff, E, (float*)out, rows, C);
     }
+    return (int)hipGetLastError();
+}
+
+int nx_clamped_glu_scale(const void* x, int is_bf16, const float* gates, long gs, int ff, int E,
+                         float limit, float slimit, float alpha, void* out, long rows, int C,
+                         hipStream_t st) {
+    if (rows * C <= 0) return 0;
+    if (E < 0 || (E > 0 && (ff <= 0 || !gates)) || (long)E * ff > C) return -1;
+    if (E == 0) ff = 8;
+    const bool vec = (C % 8) == 0 && (ff % 8) == 0 && ((uintptr_t)x % 16) == 0 &&
+                     ((uintptr_t)out % 16) == 0;
+    if (vec) {
+        dim3 grid(grid_for(rows * (C / 8), 256)), block(256);
+        if (is_bf16) clamped_glu_scale_vec_kernel<bf16><<<grid, block, 0, st>>>(
+            (const bf16*)x, gates, gs, ff, E, limit, slimit, alpha, (bf16*)out, rows, C);
+        else clamped_glu_scale_vec_kernel<float><<<grid, block, 0, st>>>(
+            (const float*)x, gates, gs, ff, E, limit, slimit, alpha, (float*)out, rows, C);
+    } else {
+        dim3 grid(grid_for(rows * C, 256)), block(256);
+        if (is_bf16) clamped_glu_scale_kernel<bf16><<<grid, block, 0, st>>>(
+            (const bf16*)x, gates, gs, ff, E, limit, slimit, alpha, (bf16*)out, rows, C);
+        else clamped_glu_scale_kernel<float><<<grid, block, 0, st>>>(
+            (const float*)x, gates, gs, ff, E, limit, slimit, alpha, (float*)out, rows, C);
+    }
+    return (int)hipGetLastError();
+}
+
+int nx_sigmoid_gate(void* y, const void* gate, long gs, int is_bf16, long rows, int C,
+                    hipStream_t st) {
+    if (rows * C <= 0) return 0;
+    const int vecn = is_bf16 ? 8 : 4;                     // elements per 16 bytes
+    const int vec = (C % 8) == 0 && (gs % vecn) == 0 && ((uintptr_t)y % 16) == 0 &&
+                    ((uintptr_t)gate % 16) == 0;
+    dim3 grid(grid_for(vec ? rows * (C / 8) : rows * C, 256)), block(256);
+    if (is_bf16) sigmoid_gate_kernel<bf16><<<grid, block, 0, st>>>(
+        (bf16*)y, (const bf16*)gate, gs, rows, C, vec);
+    else sigmoid_gate_kernel<float><<<grid, block, 0, st>>>(
+        (float*)y, (const float*)gate, gs, rows, C, vec);
     return (int)hipGetLastError();
 }
 

@@ -302,10 +302,13 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping):
 def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
                     window=None, keep_first=0, r1=None, r2=None, gate=None,
                     softcap=0.0, sink=None, q_temp=None, out_dtype=torch.float32,
-                    gate_per_head=False):
+                    gate_per_head=False, chunk=0, slopes=None):
     """Softmax attention of ragged queries against a paged cache, every
     option a parameter. Query at position i sees key j <= i when no window
-    is given, else when i-j < window or j < keep_first. Score, in order:
+    is given, else when i-j < window or j < keep_first; with ``chunk`` > 0
+    also only keys of its own block of ``chunk`` positions (floor(i/chunk)
+    = floor(j/chunk), blocks counted from position 0). ``slopes`` (H,)
+    takes slope_h * (i-j) off the score. Score, in order:
     q.k * scale * temp(i) with temp(i) = 1 + coef*ln(floor((i+1)/every)+1)
     (``q_temp`` = (coef, every)); minus r1_h*log1p(r2_h*(i-j)) when r1/r2
     are given; then softcap*tanh(score/softcap) when softcap > 0. ``sink``
@@ -337,11 +340,15 @@ def paged_attention(q, k_cache, v_cache, positions, block_table, scale,
             dist = (i - j).clamp(min=0)
             s = s - r1.float().view(1, H, 1, 1) * torch.log1p(
                 r2.float().view(1, H, 1, 1) * dist)
+        if slopes is not None:
+            s = s - slopes.float().view(1, H, 1, 1) * (i - j).clamp(min=0)
         if softcap:
             s = softcap * torch.tanh(s / softcap)
         vis = j <= i
         if window is not None:
             vis = vis & ((i - j < window) | (j < keep_first))
+        if chunk:
+            vis = vis & (torch.floor(i / chunk) == torch.floor(j / chunk))
         s = s.masked_fill(~vis, float("-inf"))
         if sink is not None:
             sk = sink.float().view(1, H, 1, 1).expand(B, H, S, 1)
@@ -540,26 +547,30 @@ def group_gated_norm(y, gate, weight, eps: float, groups: int, gate_first: bool,
 
 
 def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int,
-                         keep_groups: int, scale: float, normalize: bool = False):
+                         keep_groups: int, scale: float, normalize: bool = False,
+                         correction=None):
     """Softmax over the first ``num_experts`` columns of fp32 ``logits``
     (T, E + extra); experts form ``n_groups`` groups of neighbours, a group
     scores as its best expert and only experts of the ``keep_groups`` best
     groups compete for the ``top_k`` places. Weights are the chosen experts'
     softmax scores times ``scale`` (divided by their sum first when
-    ``normalize``). Extra columns are per-token sigmoid gates. Returns
+    ``normalize``). ``correction`` (E,) is added to the scores for the choice
+    only (the weights stay the scores). Extra columns are per-token sigmoid
+    gates. Returns
     (dense (T, E + extra) fp32 with zeros at unchosen experts, idx (T, top_k)
     int32, weights (T, top_k) fp32)."""
     T = logits.shape[0]
     E = num_experts
     lf = logits.float()
     s = torch.softmax(lf[:, :E], dim=-1)
-    cand = s
+    cand = s if correction is None else s + correction.float()
     if n_groups > 1 and keep_groups < n_groups:
         per = E // n_groups
         gs = s.view(T, n_groups, per).max(-1).values
         best = gs.topk(keep_groups, dim=-1).indices
         gmask = torch.zeros_like(gs, dtype=torch.bool).scatter(1, best, True)
-        cand = torch.where(gmask.repeat_interleave(per, dim=1), s, torch.full_like(s, -1.0))
+        cand = torch.where(gmask.repeat_interleave(per, dim=1), cand,
+                           torch.full_like(s, float("-inf")))
     idx = cand.topk(top_k, dim=-1).indices
     w = s.gather(1, idx)
     if normalize:
@@ -571,15 +582,40 @@ def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int,
     return dense, idx.to(torch.int32), w
 
 
+def clamped_glu_scale(hid, gates, expert_ff: int, num_experts: int, limit: float,
+                      shared_limit: float, alpha: float, out_dtype):
+    """Clamped gated units of stacked experts: ``hid`` (T, 2*C) holds
+    [gate | up] pre-activations of C = E*ff + rest columns; column c < E*ff
+    belongs to expert c // ff (clamp ``limit``, times the token's routing
+    weight ``gates[t, c // ff]``), the remaining columns to an always-on
+    shared expert (clamp ``shared_limit``, weight one). ``gates`` (T, >= E)
+    fp32; further columns are ignored."""
+    T, C2 = hid.shape
+    C = C2 // 2
+    E = num_experts
+    g, u = hid.float()[:, :C], hid.float()[:, C:]
+    ne = E * expert_ff
+    out = torch.empty(T, C, dtype=torch.float32, device=hid.device)
+    if ne:
+        cols = torch.arange(ne, device=hid.device) // expert_ff
+        out[:, :ne] = clamped_glu(g[:, :ne], u[:, :ne], limit, alpha) * gates.float()[:, cols]
+    if C > ne:
+        out[:, ne:] = clamped_glu(g[:, ne:], u[:, ne:], shared_limit, alpha)
+    return out.to(out_dtype)
+
+
 def relu2_scale(hid, gates, expert_ff: int, num_experts: int, out_dtype):
     """(T, E*ff + rest) hidden pre-activations -> relu(x)^2 times the token's
     gate of the column's owner: column c < E*ff belongs to expert c // ff,
     the remaining columns (a shared expert) to gate column E; ``gates`` is
-    (T, E + 1), or (T, E) when there are no remaining columns."""
+    (T, E + 1), or (T, E) when there are no remaining columns, or None for a
+    plain relu(x)^2."""
     T, C = hid.shape
     E = num_experts
-    assert C == E * expert_ff or gates.shape[1] == E + 1
     hf = torch.relu(hid.float()) ** 2
+    if gates is None:
+        return hf.to(out_dtype)
+    assert C == E * expert_ff or gates.shape[1] == E + 1
     cols = (torch.arange(C, device=hid.device) // expert_ff).clamp(max=E)
     return (hf * gates.float()[:, cols]).to(out_dtype)
 

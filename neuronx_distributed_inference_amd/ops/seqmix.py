@@ -249,11 +249,14 @@ def paged_kv_write(k_cache, v_cache, k_new, v_new, slot_mapping, step: "StepLayo
 def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: float,
                     num_heads: int, window: Optional[int] = None, keep_first: int = 0,
                     r1=None, r2=None, gate=None, softcap: float = 0.0, sink=None,
-                    q_temp=None, out_dtype=None, gate_per_head: bool = False):
+                    q_temp=None, out_dtype=None, gate_per_head: bool = False,
+                    chunk: int = 0, slopes=None):
     """q (B,S,H*Dk) (row-strided view allowed) against the paged cache ->
     (B,S,H*Dv). Options (see ref.paged_attention): sliding ``window`` with
-    ``keep_first`` always-visible tokens (None = plain causal), log-distance
-    penalty ``r1``/``r2``, tanh score cap, per-head softmax ``sink``, query
+    ``keep_first`` always-visible tokens (None = plain causal), ``chunk`` > 0
+    = only keys of the query's own block of that many positions, log-distance
+    penalty ``r1``/``r2`` or linear distance penalty ``slopes`` (H,), tanh
+    score cap, per-head softmax ``sink``, query
     temperature ``q_temp`` = (coef, every), sigmoid output ``gate``
     ((B,S,H*Dv), or (B,S,H) with ``gate_per_head``).
     ``v_cache`` may be ``k_cache[..., :Dv]`` (values inside the key rows)."""
@@ -262,10 +265,13 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
     G, Dk = k_cache.shape[2], k_cache.shape[3]
     Dv = v_cache.shape[3]
     out_dtype = out_dtype or q.dtype
+    assert slopes is None or r1 is None, "one distance penalty at a time"
     if q.is_cuda:
         lib = _load()
         out = torch.empty(B, S, H * Dv, dtype=out_dtype, device=q.device)
         bt = step.i32(block_table)
+        if slopes is not None:
+            r1, r2 = slopes, None          # the kernels read a lone r1 as slopes
         assert k_cache.stride(3) == 1 and v_cache.stride(3) == 1
         assert k_cache.stride(1) == k_cache.stride(2) * G and v_cache.stride(1) == v_cache.stride(2) * G
         assert k_cache.stride(0) == k_cache.stride(1) * k_cache.shape[1]
@@ -277,9 +283,14 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
         # and merged; the partials need a workspace
         ws, nks = None, 1
         if S == 1 and G == 1 and q.dtype == torch.bfloat16 and \
-                v_cache.data_ptr() == k_cache.data_ptr() and window is None:
+                v_cache.data_ptr() == k_cache.data_ptr():
             groups = B * ((H + 15) // 16) * ((Dv + 511) // 512)
-            nks = max(1, min(8, 256 // max(groups, 1), (bt.shape[1] * k_cache.shape[1]) // 128))
+            span = bt.shape[1] * k_cache.shape[1]           # most keys a token can see
+            if window is not None:
+                span = min(span, int(window) + 31)
+            if chunk:
+                span = min(span, int(chunk) + 31)
+            nks = max(1, min(8, 256 // max(groups, 1), span // 128))
             if nks > 1:
                 ws = torch.empty(B * H * nks * (Dv + 2), dtype=torch.float32, device=q.device)
         _check(lib.nx_paged_attn(
@@ -294,13 +305,14 @@ def paged_attention(q, k_cache, v_cache, step: StepLayout, block_table, scale: f
             k_cache.shape[1], ctypes.c_float(scale),
             int(window) if window is not None else 0x7fffffff, int(keep_first),
             ctypes.c_float(softcap or 0.0), ctypes.c_float(coef), every,
-            _p(ws), nks, int(bool(gate_per_head)), _stream()), "paged_attention")
+            _p(ws), nks, int(bool(gate_per_head)), int(chunk or 0), _stream()),
+            "paged_attention")
         return out
     return ref.paged_attention(
         q.reshape(B, S, H, Dk), k_cache, v_cache, step.positions, block_table, scale,
         window=window, keep_first=keep_first, r1=r1, r2=r2, gate=gate,
         softcap=softcap or 0.0, sink=sink, q_temp=q_temp, out_dtype=out_dtype,
-        gate_per_head=gate_per_head)
+        gate_per_head=gate_per_head, chunk=int(chunk or 0), slopes=slopes)
 
 
 def window_bias_attention(q, k_cache, v_cache, step: StepLayout, block_table,
@@ -418,28 +430,50 @@ def rms_norm(x, weight, eps: float, one_plus: bool = False, out_dtype=None, out=
     return y
 
 
-def add_rms_norm(stream, y, weight, eps: float, one_plus: bool = True, copy_dtype=None):
+def add_rms_norm(stream, y, weight, eps: float, one_plus: bool = True, copy_dtype=None,
+                 extra=None, coef=None, next_weight=None):
     """Post-norm residual step on the fp32 stream, in place:
-    stream += rms_norm(y) * (1 + w). Returns the updated stream cast to
-    ``copy_dtype`` (the next sublayer's GEMM input) or None."""
+    stream += rms_norm(y) * w (``one_plus``: * (1 + w)). With ``extra``
+    (same shape as y) and ``coef`` (rows, n) fp32, the normed vector is
+    y + sum(coef[row]) * extra[row] (experts that pass their input through).
+    Returns the updated stream cast to ``copy_dtype`` (the next sublayer's
+    GEMM input), or, with ``next_weight``, the next sublayer's pre-norm
+    rms_norm(stream) * next_weight in ``copy_dtype``; None without a
+    ``copy_dtype``."""
+    assert (extra is None) == (coef is None)
     if stream.is_cuda:
         lib = _load()
         assert stream.dtype == torch.float32 and stream.is_contiguous()
         y = y.contiguous()
         C = stream.shape[-1]
+        rows = stream.numel() // C
         copy = None
-        if copy_dtype is not None and copy_dtype != torch.float32:
+        if copy_dtype is not None and (copy_dtype != torch.float32 or next_weight is not None):
             copy = torch.empty(stream.shape, dtype=copy_dtype, device=stream.device)
+        nc, cs = 0, 0
+        if extra is not None:
+            extra = extra.contiguous()
+            assert extra.dtype == y.dtype and extra.numel() == y.numel()
+            assert coef.dtype == torch.float32 and coef.stride(-1) == 1 and coef.dim() == 2
+            assert coef.shape[0] == rows
+            nc, cs = coef.shape[1], coef.stride(0)
         _check(lib.nx_add_rms_norm(
             _p(stream), _p(y), _is_bf16(y), _p(_f32(weight)), int(one_plus),
-            ctypes.c_float(eps), _p(copy), ctypes.c_long(stream.numel() // C), C,
-            _stream()), "add_rms_norm")
-        if copy_dtype == torch.float32:
+            ctypes.c_float(eps), _p(copy), 0 if copy is None else _is_bf16(copy),
+            _p(extra), _p(coef), ctypes.c_long(cs), nc,
+            _p(None if next_weight is None else _f32(next_weight)),
+            ctypes.c_long(rows), C, _stream()), "add_rms_norm")
+        if copy_dtype == torch.float32 and next_weight is None:
             return stream
         return copy
-    stream.add_(ref.rms_norm_rows(y, weight, eps, one_plus, torch.float32))
+    v = y.float()
+    if extra is not None:
+        v = v + coef.float().sum(-1).view(*y.shape[:-1], 1) * extra.float()
+    stream.add_(ref.rms_norm_rows(v, weight, eps, one_plus, torch.float32))
     if copy_dtype is None:
         return None
+    if next_weight is not None:
+        return ref.rms_norm_rows(stream, next_weight, eps, False, copy_dtype)
     return stream if copy_dtype == torch.float32 else stream.to(copy_dtype)
 
 
@@ -585,9 +619,11 @@ def group_gated_norm(y, gate, weight, eps: float, groups: int, gate_first: bool,
 
 
 def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int = 1,
-                         keep_groups: int = 1, scale: float = 1.0, normalize: bool = False):
+                         keep_groups: int = 1, scale: float = 1.0, normalize: bool = False,
+                         correction=None):
     """Group-limited top-k routing on fp32 logits (T, E + extra) (see
-    ref.group_limited_router): returns (dense (T, E + extra) weights with
+    ref.group_limited_router; ``correction`` (E,) shifts the scores for the
+    choice only): returns (dense (T, E + extra) weights with
     sigmoid gates in the extra columns, idx (T, top_k) int32, weights)."""
     if logits.is_cuda:
         lib = _load()
@@ -601,29 +637,75 @@ def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int = 1
         _check(lib.nx_group_router(
             _p(logits), ctypes.c_long(logits.stride(0)), E, C - E, top_k, max(n_groups, 1),
             max(min(keep_groups, n_groups), 1), ctypes.c_float(scale), int(normalize),
+            _p(None if correction is None else _f32(correction)),
             _p(dense), _p(idx), _p(wts), ctypes.c_long(T), _stream()), "group_limited_router")
         return dense, idx, wts
     return ref.group_limited_router(logits, num_experts, top_k, max(n_groups, 1),
-                                    max(min(keep_groups, n_groups), 1), scale, normalize)
+                                    max(min(keep_groups, n_groups), 1), scale, normalize,
+                                    correction)
 
 
 def relu2_scale(hid, gates, expert_ff: int, num_experts: int, out_dtype=None):
     """relu(x)^2 of (T, E*ff + rest) pre-activations times the token's gate of
     the column's expert; the remaining columns take gate column E (see
-    ref.relu2_scale)."""
+    ref.relu2_scale). ``gates`` None: plain relu(x)^2."""
     out_dtype = out_dtype or hid.dtype
     if hid.is_cuda:
         lib = _load()
         T, C = hid.shape
-        assert hid.is_contiguous() and gates.dtype == torch.float32 and gates.is_contiguous()
-        assert out_dtype == hid.dtype
-        assert C == num_experts * expert_ff or gates.shape[1] == num_experts + 1
+        assert hid.is_contiguous() and out_dtype == hid.dtype
         out = torch.empty(T, C, dtype=out_dtype, device=hid.device)
+        if gates is None:
+            _check(lib.nx_relu2_scale(_p(hid), _is_bf16(hid), _p(None), 0, max(C, 1), 1,
+                                      _p(out), ctypes.c_long(T), C, _stream()), "relu2_scale")
+            return out
+        assert gates.dtype == torch.float32 and gates.is_contiguous()
+        assert C == num_experts * expert_ff or gates.shape[1] == num_experts + 1
         _check(lib.nx_relu2_scale(_p(hid), _is_bf16(hid), _p(gates), gates.shape[1], expert_ff,
                                   num_experts, _p(out), ctypes.c_long(T), C, _stream()),
                "relu2_scale")
         return out
     return ref.relu2_scale(hid, gates, expert_ff, num_experts, out_dtype)
+
+
+def clamped_glu_scale(hid, gates, expert_ff: int, num_experts: int, limit: float,
+                      shared_limit: float = 0.0, alpha: float = 1.702, out_dtype=None):
+    """Clamped gated units of stacked experts (see ref.clamped_glu_scale):
+    hid (T, 2*C) = [gate | up] of C = E*ff + shared columns -> (T, C), an
+    expert's columns times the token's routing weight ``gates[t, e]`` (fp32,
+    (T, >= E), row-strided), the shared columns with their own clamp."""
+    out_dtype = out_dtype or hid.dtype
+    if hid.is_cuda:
+        lib = _load()
+        T, C2 = hid.shape
+        C = C2 // 2
+        assert hid.is_contiguous() and out_dtype == hid.dtype and C2 == 2 * C
+        assert num_experts * expert_ff <= C
+        if num_experts:
+            assert gates.dtype == torch.float32 and gates.stride(1) == 1
+            assert gates.shape[0] == T and gates.shape[1] >= num_experts
+        out = torch.empty(T, C, dtype=out_dtype, device=hid.device)
+        _check(lib.nx_clamped_glu_scale(
+            _p(hid), _is_bf16(hid), _p(gates if num_experts else None),
+            ctypes.c_long(gates.stride(0) if num_experts else 0), expert_ff, num_experts,
+            ctypes.c_float(limit), ctypes.c_float(shared_limit), ctypes.c_float(alpha),
+            _p(out), ctypes.c_long(T), C, _stream()), "clamped_glu_scale")
+        return out
+    return ref.clamped_glu_scale(hid, gates, expert_ff, num_experts, limit, shared_limit,
+                                 alpha, out_dtype)
+
+
+def sigmoid_gate_(y, gate):
+    """In place: y *= sigmoid(gate). y (..., C) contiguous; ``gate`` of the
+    same shape may be a column slice of a wider tensor."""
+    if y.is_cuda:
+        lib = _load()
+        C = y.shape[-1]
+        assert y.is_contiguous() and gate.shape == y.shape and gate.dtype == y.dtype
+        _check(lib.nx_sigmoid_gate(_p(y), _p(gate), ctypes.c_long(_rows_view(gate)), _is_bf16(y),
+                                   ctypes.c_long(y.numel() // C), C, _stream()), "sigmoid_gate")
+        return y
+    return y.copy_(y.float() * torch.sigmoid(gate.float()))
 
 
 def scaled_residual(x, terms, eps: float = 0.0):

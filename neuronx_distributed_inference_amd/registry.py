@@ -76,6 +76,11 @@ _REGISTRY: Dict[str, Tuple[str, str, str]] = {
         "KuteraxInferenceConfig",
         "KuteraxForCausalLM",
     ),
+    "tamilix": (
+        "neuronx_distributed_inference_amd.models.tamilix.modeling_tamilix",
+        "TamilixInferenceConfig",
+        "TamilixForCausalLM",
+    ),
     "soputar": (
         "neuronx_distributed_inference_amd.models.soputar.modeling_soputar",
         "SoputarInferenceConfig",
