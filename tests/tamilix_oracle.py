@@ -92,19 +92,17 @@ def attention_mixer(h, weights, pre, mc):
     return out.reshape(T, H * Dv) @ _w(weights, pre + "o").T
 
 
-def latent_mixer(h, weights, pre, mc, eps):
-    """Latent attention: queries through a normed latent, keys and values
-    expanded from a normed latent, one rotated key part for all heads, a
-    sliding window, an element-wise sigmoid gate. h (T, W)."""
-    T = h.shape[0]
+def latent_attend(q, dkv, weights, pre, mc, eps):
+    """The attention of the latent mixer from its projections: q (T, H *
+    (dim + rot_dim)) after the query up-projection, dkv (T, kv_rank +
+    rot_dim) before the latent's norm. Returns the concatenated heads."""
+    T = q.shape[0]
     H, D, R, Dv, C = mc["heads"], mc["dim"], mc["rot_dim"], mc["vdim"], mc["kv_rank"]
     rot = mc["rot"]
     pos = torch.arange(T)
-    cq = norm(h @ _w(weights, pre + "dq").T, _w(weights, pre + "dq.norm"), eps)
-    q = (cq @ _w(weights, pre + "uq").T).view(T, H, D + R)
-    dkv = h @ _w(weights, pre + "dkv").T
+    q = q.view(T, H, D + R)
     c = norm(dkv[:, :C], _w(weights, pre + "dkv.norm"), eps)
-    k_rot = rotate_pairs(dkv[:, C:].view(T, 1, R), pos, rot["base"], rot["dims"])[:, 0]
+    k_rot = rotate_pairs(dkv[:, C:].reshape(T, 1, R), pos, rot["base"], rot["dims"])[:, 0]
     q_rot = rotate_pairs(q[..., D:], pos, rot["base"], rot["dims"])
     k_plain = (c @ _w(weights, pre + "uk").T).view(T, H, D)
     v = (c @ _w(weights, pre + "uv").T).view(T, H, Dv)
@@ -113,8 +111,19 @@ def latent_mixer(h, weights, pre, mc, eps):
     for hd in range(H):
         s = (q[:, hd, :D] @ k_plain[:, hd].T + q_rot[:, hd] @ k_rot.T) * mc["scale"]
         out[:, hd] = sink_softmax(s, vis) @ v[:, hd]
+    return out.reshape(T, H * Dv)
+
+
+def latent_mixer(h, weights, pre, mc, eps):
+    """Latent attention: queries through a normed latent, keys and values
+    expanded from a normed latent, one rotated key part for all heads, a
+    sliding window, an element-wise sigmoid gate. h (T, W)."""
+    cq = norm(h @ _w(weights, pre + "dq").T, _w(weights, pre + "dq.norm"), eps)
+    q = cq @ _w(weights, pre + "uq").T
+    dkv = h @ _w(weights, pre + "dkv").T
+    heads = latent_attend(q, dkv, weights, pre, mc, eps)
     gate = torch.sigmoid(h @ _w(weights, pre + "g").T)
-    return (out.reshape(T, H * Dv) * gate) @ _w(weights, pre + "o").T
+    return (heads * gate) @ _w(weights, pre + "o").T
 
 
 def dense_ff(h, weights, pre):
