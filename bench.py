@@ -72,10 +72,12 @@ def parse_args():
                    help="prefill/decode throughput of the hybrid decoders (Nabelix: windowed "
                         "attention + gated delta rule; Soputar: latent, delta-rule and capped "
                         "attention layers; Kuterax: sink attention + state space in "
-                        "parallel, retention, routed experts) beside Llama at equal "
-                        "width/depth/ff/vocab")
-    p.add_argument("--hybrid-models", default="llama,nabelix,soputar,kuterax",
-                   help="comma-separated subset of llama,nabelix,soputar,kuterax for --hybrid")
+                        "parallel, retention, routed experts; Tamilix: chunk-local slope "
+                        "attention, windowed gated latent attention, identity-routed "
+                        "experts) beside Llama at equal width/depth/ff/vocab")
+    p.add_argument("--hybrid-models", default="llama,nabelix,soputar,kuterax,tamilix",
+                   help="comma-separated subset of llama,nabelix,soputar,kuterax,tamilix "
+                        "for --hybrid")
     p.add_argument("--hybrid-sizes", default="2048,4096",
                    help="comma-separated layer widths for --hybrid")
     p.add_argument("--hybrid-layers", type=int, default=4)
@@ -114,6 +116,9 @@ def run_hybrid_bench(args):
     )
     from neuronx_distributed_inference_amd.models.kuterax.modeling_kuterax import (
         KuteraxForCausalLM, KuteraxInferenceConfig,
+    )
+    from neuronx_distributed_inference_amd.models.tamilix.modeling_tamilix import (
+        TamilixForCausalLM, TamilixInferenceConfig,
     )
 
     dtype = "bfloat16" if on_gpu else "float32"
@@ -192,6 +197,40 @@ def run_hybrid_bench(args):
                 max_positions=max_len, layers=[par if i % 2 == 0 else ret for i in range(L)],
                 loop={"start": 0, "stop": L, "times": 1}, norm={"eps": 1e-5})
             cls = KuteraxForCausalLM
+        elif kind == "tamilix":
+            # the design's layer mix, repeated to depth L: chunk-local slope
+            # attention with a dense relu-squared feed-forward, windowed latent
+            # attention (512-wide latent + 64 rotated channels, query latent of
+            # 3/4 width) with routed experts, attention with routed experts, and
+            # a latent layer that runs the second layer's weights again. The
+            # routed feed-forward activates at most ff columns per token: four
+            # of sixteen experts of ff/8 and two pass-through experts, plus a
+            # shared expert of ff/2
+            moe = {"kind": "moe", "expert": {"ff": ff // 8, "limit": 7.0},
+                   "shared": {"ff": ff // 2, "limit": 7.0},
+                   "router": {"experts": 16, "identity": 2, "top": 4}}
+            att = {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                   "mask": {"size": 1024}}
+            lat = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128,
+                   "kv_rank": min(512, width // 4), "q_rank": width * 3 // 4,
+                   "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64},
+                   "mask": {"size": 1024}}
+            quad = [
+                {"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": ff}},
+                {"type": "latent_attention", "mixer": lat, "mlp": moe},
+                {"type": "attention", "mixer": att, "mlp": moe},
+                {"type": "latent_attention", "mixer": lat, "mlp": moe, "weights_of": 1},
+            ]
+            layers = []
+            for i in range(L):
+                lc = json.loads(json.dumps(quad[i % 4]))
+                if "weights_of" in lc:
+                    lc["weights_of"] = i - 2
+                layers.append(lc)
+            cfg = TamilixInferenceConfig(
+                neuron_config=ec, architecture="Tamilix", width=width, vocab=V,
+                layers=layers, norm={"eps": 1e-5}, embedding={"scale": 8.0})
+            cls = TamilixForCausalLM
         else:
             layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff}, "mixer": {
                 "left": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128,
@@ -219,7 +258,7 @@ def run_hybrid_bench(args):
         return m
 
     for width in [int(x) for x in args.hybrid_sizes.split(",")]:
-        for kind in [k for k in ("llama", "nabelix", "soputar", "kuterax")
+        for kind in [k for k in ("llama", "nabelix", "soputar", "kuterax", "tamilix")
                      if k in args.hybrid_models.split(",")]:
             with torch.inference_mode():
                 # ---- prefill: one prompt, three timed repetitions

@@ -821,10 +821,14 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, long qstride, const bf16* __r
                     k_lds + (kb * 16 + lr) * KS + ks * 32 + lg * 8);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[ks], acc, 0, 0, 0);
             }
-            if (whole && !r1) {                          // uniform
+            if (whole && !r2) {                          // uniform
+                // (a linear penalty needs no mask either: the tile's keys are
+                // lo + base + 16 kb + 4 lg + r, all at or before every row)
+                const float d0 = (float)(my_i - (lo + base + kb * 16 + lg * 4));
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float x = acc[r] * qscale;
+                    if (r1) x -= a1 * (d0 - (float)r);
                     if (cap > 0.f) x = cap * fast_tanh_(x / cap);
                     if (my_i < 0) x = -INFINITY;
                     sv[kb][r] = x;

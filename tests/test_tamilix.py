@@ -461,8 +461,24 @@ def test_chunked_attention_far_key_among_hundreds(device, cuts):
 def test_chunked_attention_bf16_matrix_path_gpu(L, cuts):
     c = L["mask"]["size"]
     spikes = [(129, (129 // c) * c), (129, (129 // c) * c - 1), (2 * c - 1, c), (c, c - 1)]
+    spikes = [(i, j) for i, j in spikes if i < 130]
     _chunked_alone("cuda", L, 130, spikes, cuts=cuts, page=16, dtype=BF16, tol=0.03, gain=3.0)
     _chunked_alone("cuda", L, 130, spikes, cuts=[100] + [1] * 30, page=16, dtype=BF16, tol=0.03,
+                   gain=3.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L", [attn_cfg(8, 4, 64, 64, scale=0.125, chunk=256),
+                               attn_cfg(16, 4, 128, 128, scale=0.09, chunk=150)])
+def test_chunked_attention_bf16_fully_visible_tiles_gpu(L):
+    """Blocks much longer than a key tile: most tiles are visible to every
+    query row of a workgroup and take the unmasked path, which still has to
+    apply the distance penalty."""
+    c = L["mask"]["size"]
+    spikes = [(329, c), (329, c - 1), (c + 100, c + 3), (c - 1, 0), (2 * c - 1 if 2 * c <= 330
+                                                                      else 300, c)]
+    _chunked_alone("cuda", L, 330, spikes, page=16, dtype=BF16, tol=0.03, gain=3.0)
+    _chunked_alone("cuda", L, 330, spikes, cuts=[200, 100, 29, 1], page=16, dtype=BF16, tol=0.03,
                    gain=3.0)
 
 
