@@ -7,8 +7,9 @@ position 0 (query ``i`` sees key ``j <= i`` only when ``floor(i / chunk) ==
 floor(j / chunk)``, wherever a prompt was cut for processing), and the
 score, from which ``slope_h * (i - j)`` is taken off. The slopes are a fixed
 geometric ladder over the heads, ``slope_h = 2^(-slope_log2 * (h + 1) / H)``.
-The softmax denominator carries one extra term ``exp(sink_h)`` per head: a
-learned key without a value that is not scaled and gets no penalty. Chunk
+The softmax denominator carries one extra term ``exp(sink_h)`` per head, a
+learned score that stands for no key: nothing is added to the output for it
+and neither the scale nor the penalty applies to it. Chunk
 size, scale, the ladder's exponent and the presence of the sink are
 constructor parameters; key and value heads may have different sizes.
 
