@@ -84,16 +84,19 @@ class TamilixInferenceConfig(InferenceConfig):
         self.num_hidden_layers = len(self.layers)
         self.tie_word_embeddings = False
         for i, lc in enumerate(self.layers):
+            if lc.get("weights_of") is not None:
+                oc = self.layers[self._owner(i)]         # what the entry omits is the owner's
+                for key in ("type", "mixer", "mlp"):
+                    if key not in lc:
+                        lc[key] = oc.get(key)
+        for i, lc in enumerate(self.layers):
             if lc.get("type") not in MIXER_TYPES:
                 raise ValueError(f"unknown Tamilix layer type {lc.get('type')!r}")
             fc = lc.get("mlp")
             if fc and fc.get("kind") not in FF_KINDS:
                 raise ValueError(f"unknown Tamilix feed-forward kind {fc.get('kind')!r}")
-            j = lc.get("weights_of")
-            if j is not None:
-                if not (isinstance(j, int) and 0 <= j < len(self.layers)) or j == i or \
-                        self.layers[j].get("weights_of") is not None:
-                    raise ValueError(f"layer {i}: weights_of must name a layer with tensors")
+            if lc.get("weights_of") is not None:
+                j = self._owner(i)
                 oc = self.layers[j]
                 if oc["type"] != lc["type"] or oc["mixer"] != lc["mixer"] or \
                         oc.get("mlp") != lc.get("mlp"):
@@ -107,10 +110,21 @@ class TamilixInferenceConfig(InferenceConfig):
             raise ValueError("Tamilix runs with tp_degree=1")
         ec.is_block_kv_layout = True
 
+    def _owner(self, i: int) -> int:
+        """Index of the entry whose tensors entry i uses (an entry that names
+        a sharing entry uses that one's owner)."""
+        seen = {i}
+        while self.layers[i].get("weights_of") is not None:
+            j = self.layers[i]["weights_of"]
+            if not (isinstance(j, int) and 0 <= j < len(self.layers)) or j in seen:
+                raise ValueError(f"layer {i}: weights_of must name a layer with tensors")
+            seen.add(j)
+            i = j
+        return i
+
     def owners(self) -> List[int]:
         """For every layer entry, the index of the entry whose tensors it uses."""
-        return [i if lc.get("weights_of") is None else lc["weights_of"]
-                for i, lc in enumerate(self.layers)]
+        return [self._owner(i) for i in range(len(self.layers))]
 
     @classmethod
     def from_hf_config(cls, model_path: str, neuron_config=None, **overrides):
@@ -134,8 +148,15 @@ class TamilixInferenceConfig(InferenceConfig):
                     hf.setdefault("vocab", emb[0])
                     hf.setdefault("width", emb[1])
                 for i, lc in enumerate(hf["layers"]):
-                    j = lc.get("weights_of")
-                    src = i if j is None else j
+                    src, seen = i, set()
+                    while isinstance(hf["layers"][src].get("weights_of"), int) and \
+                            src not in seen and 0 <= hf["layers"][src]["weights_of"] < len(hf["layers"]):
+                        seen.add(src)
+                        src = hf["layers"][src]["weights_of"]
+                    if src != i:
+                        for key in ("type", "mixer", "mlp"):
+                            if key not in lc:
+                                lc[key] = json.loads(json.dumps(hf["layers"][src].get(key)))
                     _fill_from_shapes(lc, lambda n, src=src: shape(f"l{src}.{n}"))
         return cls(neuron_config=neuron_config, **hf)
 

@@ -475,8 +475,7 @@ def test_chunked_attention_bf16_fully_visible_tiles_gpu(L):
     query row of a workgroup and take the unmasked path, which still has to
     apply the distance penalty."""
     c = L["mask"]["size"]
-    spikes = [(329, c), (329, c - 1), (c + 100, c + 3), (c - 1, 0), (2 * c - 1 if 2 * c <= 330
-                                                                      else 300, c)]
+    spikes = [(329, c), (329, c - 1), (c + 60, c + 3), (c - 1, 0), (min(2 * c - 1, 300), c)]
     _chunked_alone("cuda", L, 330, spikes, page=16, dtype=BF16, tol=0.03, gain=3.0)
     _chunked_alone("cuda", L, 330, spikes, cuts=[200, 100, 29, 1], page=16, dtype=BF16, tol=0.03,
                    gain=3.0)
@@ -715,6 +714,22 @@ def test_residual_stream_per_layer_run(device, make):
         close(s[0], streams[r], 1e-4)
 
 
+def test_sharing_entries_may_chain_and_omit_what_equals_the_owner():
+    cfg = model_cfg()
+    W = make_weights(cfg, seed=18)
+    toks = tokens_for(cfg, 14, seed=19)
+    want = oracle.forward(cfg, W, toks)
+    short = copy.deepcopy(cfg)
+    short["layers"][3] = {"type": "latent_attention", "weights_of": 1}
+    short["layers"].append({"weights_of": 3})            # through layer 3 to layer 1
+    full = copy.deepcopy(cfg)
+    full["layers"].append(copy.deepcopy(full["layers"][3]))
+    eng = make_engine(short, W)
+    assert eng.model.model._order_slots == [0, 1, 2, 1, 1]
+    close(feed(eng, toks, [9, 5]), oracle.forward(full, W, toks), 3e-4)
+    assert not torch.allclose(oracle.forward(full, W, toks), want)
+
+
 def test_shared_weights_keep_their_own_cache():
     """A layer with weights_of has no parameters but pages of its own: the
     two runs of one module see different keys."""
@@ -932,7 +947,7 @@ def test_config_rejects_what_it_does_not_know():
     for change in (lambda c: c["layers"][1].update(type="window"),
                    lambda c: c["layers"][0]["mlp"].update(kind="experts"),
                    lambda c: c["layers"][3].update(weights_of=3),        # itself
-                   lambda c: c["layers"][2].update(weights_of=3),        # a layer without tensors
+                   lambda c: c["layers"][3].update(weights_of=9),        # no such layer
                    lambda c: c["layers"][3].update(weights_of=0),        # another kind of layer
                    lambda c: c["layers"][1]["mlp"]["router"].update(top=9)):
         bad = copy.deepcopy(cfg)
