@@ -84,16 +84,16 @@ class LatentSinkAttention(nn.Module):
         H, D, R, C = self.num_heads, self.dim, self.rot_dim, self.kv_rank
         T = B * S
         dt = q.dtype
-        # cache row [rms_norm(latent) | rotated shared key part]
-        row = torch.empty(B, S, self.row, dtype=dt, device=q.device)
-        self.latent_norm(dkv[..., :C], out=row[..., :C])
-        seqmix.rotate_interleaved(dkv[..., C:].unsqueeze(2), step, self.inv_freq,
-                                  out=row[..., C:].unsqueeze(2))
+        # cache row [rms_norm(latent) | rotated shared key part], normed, rotated
+        # and scattered to the token's page slot in one launch; only the
+        # whole-prompt form reads it back as a dense tensor
         kc, _ = kv_mgr.get_cache(cache_idx)
-        seqmix.paged_kv_write(kc.data, None, row.view(T, self.row), None,
-                              kv_mgr.slot_mapping, step)
         q4 = q.unflatten(-1, (H, D + R))
-        if getattr(step, "fresh", False):
+        fresh = bool(getattr(step, "fresh", False))
+        row = torch.empty(B, S, self.row, dtype=dt, device=q.device) if fresh else None
+        seqmix.latent_row_write(dkv, self.latent_norm.weight, self.latent_norm.eps,
+                                self.inv_freq, step, kc.data, kv_mgr.slot_mapping, C, row=row)
+        if fresh:
             return self._expanded(q4, row, step, gate)
         # query in latent space: [uk_h^T q_plain | rotated q_rot] per head
         qa = torch.empty(B, S, H, self.row, dtype=dt, device=q.device)

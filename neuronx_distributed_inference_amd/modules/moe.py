@@ -430,10 +430,9 @@ class GroupLimitedRouter(nn.Module):
         weights (T, top_k) fp32)."""
         from neuronx_distributed_inference_amd.ops import seqmix
 
-        logits = F.linear(x.float(), self.weight)
-        return seqmix.group_limited_router(logits, self.num_experts, self.top_k, self.n_groups,
-                                           self.keep_groups, self.scale, self.normalize,
-                                           correction=self.correction)
+        return seqmix.route_tokens(x, self.weight, self.num_experts, self.top_k, self.n_groups,
+                                   self.keep_groups, self.scale, self.normalize,
+                                   correction=self.correction)
 
 
 class FusedUngatedExperts(nn.Module):

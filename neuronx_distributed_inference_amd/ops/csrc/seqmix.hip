@@ -283,6 +283,51 @@ __global__ void paged_kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc,
     }
 }
 
+// --------------------------------------------- latent cache row, one launch
+// A latent layer's cache row of a token: [rms_norm(x[:C]) * w | x[C:C+R] with its
+// first 2*half channels turned in interleaved pairs by pos * inv_freq[i]], written
+// straight into the token's page slot (and, when `row` is given, into a dense row
+// buffer as well). One wave per token; statistics and angles in fp32. Pad tokens
+// (slot or position < 0) write nothing to the cache.
+template <typename T>
+__global__ void latent_row_kernel(const T* __restrict__ x, long xs, const float* __restrict__ w,
+                                  float eps, const float* __restrict__ inv_freq, int half,
+                                  const int* __restrict__ pos, const int* __restrict__ slots,
+                                  T* __restrict__ cache, long nslots, T* __restrict__ row, long rs,
+                                  long ntok, int C, int R) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long tok = (long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (tok >= ntok) return;
+    const int s = slots[tok], p = pos[tok];
+    T* cp = (s >= 0 && s < nslots && p >= 0) ? cache + (long)s * (C + R) : nullptr;
+    T* rp = row ? row + tok * rs : nullptr;
+    if (!cp && !rp) return;
+    const T* xr = x + tok * xs;
+    float ss = 0.f;
+    for (int c = lane; c < C; c += WAVE) { const float v = ldf<T>(xr + c); ss += v * v; }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / C + eps);
+    for (int c = lane; c < C; c += WAVE) {
+        const float v = ldf<T>(xr + c) * inv * w[c];
+        if (cp) stf<T>(cp + c, v);
+        if (rp) stf<T>(rp + c, v);
+    }
+    for (int e = lane; e < half + (R - 2 * half); e += WAVE) {
+        if (e < half) {
+            const float a = ldf<T>(xr + C + 2 * e), b = ldf<T>(xr + C + 2 * e + 1);
+            float sn, cs;
+            sincosf((float)(p < 0 ? 0 : p) * inv_freq[e], &sn, &cs);
+            const float u = a * cs - b * sn, v = b * cs + a * sn;
+            if (cp) { stf<T>(cp + C + 2 * e, u); stf<T>(cp + C + 2 * e + 1, v); }
+            if (rp) { stf<T>(rp + C + 2 * e, u); stf<T>(rp + C + 2 * e + 1, v); }
+        } else {
+            const int c = C + 2 * half + (e - half);
+            const float v = ldf<T>(xr + c);
+            if (cp) stf<T>(cp + c, v);
+            if (rp) stf<T>(rp + c, v);
+        }
+    }
+}
+
 // ----------------------------------------------------------- paged attention
 // Score of query i and key j, in order: q.k * scale * temp(i), temp(i) = 1 +
 // qt_coef * ln(floor((i+1)/qt_every) + 1) (qt_every = 0: none); minus
@@ -2038,20 +2083,15 @@ DEV void wave_argmax(float& v, int& i) {
 }
 
 #define RT_WAVES 4
-__global__ void __launch_bounds__(RT_WAVES * WAVE)
-group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra, int top,
-                    int ngroups, int keep, float scale, int normalize,
-                    const float* __restrict__ corr,
-                    float* __restrict__ dense, int* __restrict__ idx, float* __restrict__ wts,
-                    long T) {
-    extern __shared__ float rsm[];                // per wave: E choice scores + ngroups + E scores
-    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
-    const long t = (long)blockIdx.x * RT_WAVES + wv;
-    if (t >= T) return;
-    float* cand = rsm + (long)wv * (2 * E + ngroups);
+// one wave: logits `lp` (E + extra, global or LDS) of a token -> its dense row
+// `dp`, chosen indices `idx` and weights `wts`; `cand` is 2E + ngroups floats of
+// LDS scratch
+DEV void route_select_(const float* lp, int E, int extra, int top, int ngroups, int keep,
+                       float scale, int normalize, const float* __restrict__ corr, float* cand,
+                       float* __restrict__ dp, int* __restrict__ idx, float* __restrict__ wts,
+                       int lane) {
     float* gsc = cand + E;
     float* sco = gsc + ngroups;                   // the uncorrected scores (the weights)
-    const float* lp = logits + t * ls;
     float m = -INFINITY;
     for (int e = lane; e < E; e += WAVE) m = fmaxf(m, lp[e]);
     m = wave_max(m);
@@ -2059,7 +2099,6 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
     for (int e = lane; e < E; e += WAVE) { const float x = expf(lp[e] - m); cand[e] = x; sum += x; }
     sum = wave_sum(sum);
     const float rs = 1.f / sum;
-    float* dp = dense + t * (long)(E + extra);
     for (int e = lane; e < E; e += WAVE) {
         const float sc = cand[e] * rs;
         sco[e] = sc;
@@ -2104,7 +2143,7 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
         if (lane == 0) cand[bi] = -INFINITY;
         if (lane == (r & (WAVE - 1))) {
             // more than 64 choices: flush the previous one first
-            if (r >= WAVE) { idx[t * top + r - WAVE] = myi; wts[t * top + r - WAVE] = myw; }
+            if (r >= WAVE) { idx[r - WAVE] = myi; wts[r - WAVE] = myw; }
             myw = bv; myi = bi;
         }
         wsum += bv;
@@ -2113,11 +2152,88 @@ group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra,
     const float f = normalize ? scale / wsum : scale;
     if (top <= WAVE) {
         if (lane < top) {
-            idx[t * top + lane] = myi;
-            wts[t * top + lane] = myw * f;
+            idx[lane] = myi;
+            wts[lane] = myw * f;
             dp[myi] = myw * f;
         }
     }
+}
+
+__global__ void __launch_bounds__(RT_WAVES * WAVE)
+group_router_kernel(const float* __restrict__ logits, long ls, int E, int extra, int top,
+                    int ngroups, int keep, float scale, int normalize,
+                    const float* __restrict__ corr,
+                    float* __restrict__ dense, int* __restrict__ idx, float* __restrict__ wts,
+                    long T) {
+    extern __shared__ float rsm[];                // per wave: E choice scores + ngroups + E scores
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x / WAVE;
+    const long t = (long)blockIdx.x * RT_WAVES + wv;
+    if (t >= T) return;
+    route_select_(logits + t * ls, E, extra, top, ngroups, keep, scale, normalize, corr,
+                  rsm + (long)wv * (2 * E + ngroups), dense + t * (long)(E + extra),
+                  idx + t * top, wts + t * top, lane);
+}
+
+// Steps of few tokens: the router's product and its selection in one launch. One
+// workgroup per token. The E + extra rows of the fp32 router weight are taken
+// eight at a time: a thread reads its 8 channels of the token's input (widened to
+// fp32) once and the same channels of the eight rows, all loads independent; the
+// eight partial dot products are summed over the wave and over the four waves
+// through LDS. The logits meet in LDS and the first wave selects as above.
+template <typename T>
+__global__ void __launch_bounds__(RT_WAVES * WAVE)
+router_fused_kernel(const T* __restrict__ x, long xs, const float* __restrict__ w, int W, int vec,
+                    int E, int extra, int top, int ngroups, int keep, float scale, int normalize,
+                    const float* __restrict__ corr, float* __restrict__ dense,
+                    int* __restrict__ idx, float* __restrict__ wts) {
+    extern __shared__ float rsm[];                // E + extra logits, then the selection scratch
+    __shared__ float part[RT_WAVES][8];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
+    const long t = blockIdx.x;
+    const T* xr = x + t * xs;
+    const int rows = E + extra;
+    for (int e0 = 0; e0 < rows; e0 += 8) {
+        float acc[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+        if (vec) {
+            for (int c = tid * 8; c < W; c += RT_WAVES * WAVE * 8) {
+                float xv[8];
+                load8<T>(xr + c, xv);
+                float wv8[8][8];                         // rows past the last repeat it
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    load8<float>(w + (long)min(e0 + k, rows - 1) * W + c, wv8[k]);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[k] += xv[j] * wv8[k][j];
+            }
+        } else {
+            for (int c = tid; c < W; c += RT_WAVES * WAVE) {
+                const float xv = ldf<T>(xr + c);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (e0 + k < rows) acc[k] += xv * w[(long)(e0 + k) * W + c];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float v = wave_sum(acc[k]);
+            if (lane == 0) part[wv][k] = v;
+        }
+        __syncthreads();
+        if (tid < 8 && e0 + tid < rows) {
+            float v = 0.f;
+#pragma unroll
+            for (int q = 0; q < RT_WAVES; ++q) v += part[q][tid];
+            rsm[e0 + tid] = v;
+        }
+        __syncthreads();
+    }
+    if (wv != 0) return;
+    route_select_(rsm, E, extra, top, ngroups, keep, scale, normalize, corr, rsm + E + extra,
+                  dense + t * (long)(E + extra), idx + t * top, wts + t * top, lane);
 }
 
 // -------------------------------------------------- relu^2 times routing weight
@@ -2816,6 +2932,42 @@ int nx_group_router(const float* logits, long ls, int E, int extra, int top, int
     dim3 grid((unsigned)((T + RT_WAVES - 1) / RT_WAVES)), block(RT_WAVES * WAVE);
     group_router_kernel<<<grid, block, sh, st>>>(logits, ls, E, extra, top, ngroups, keep, scale,
                                                  normalize, corr, dense, idx, wts, T);
+    return (int)hipGetLastError();
+}
+
+int nx_router_fused(const void* x, long xs, int x_bf16, const float* w, int W, int E, int extra,
+                    int top, int ngroups, int keep, float scale, int normalize, const float* corr,
+                    float* dense, int* idx, float* wts, long T, hipStream_t st) {
+    if (T <= 0) return 0;
+    if (E <= 0 || top <= 0 || top > E || top > WAVE || ngroups <= 0 || E % ngroups != 0 ||
+        keep <= 0 || keep > ngroups || (long)top > (long)(E / ngroups) * keep || W <= 0) return -1;
+    const size_t sh = (size_t)(3 * E + extra + ngroups) * sizeof(float);
+    if (sh > 60 * 1024) return -2;
+    const int vecn = x_bf16 ? 8 : 4;
+    const int vec = (W % 8) == 0 && (xs % vecn) == 0 && ((uintptr_t)x % 16) == 0 &&
+                    ((uintptr_t)w % 16) == 0;
+    dim3 grid((unsigned)T), block(RT_WAVES * WAVE);
+    if (x_bf16) router_fused_kernel<bf16><<<grid, block, sh, st>>>(
+        (const bf16*)x, xs, w, W, vec, E, extra, top, ngroups, keep, scale, normalize, corr, dense,
+        idx, wts);
+    else router_fused_kernel<float><<<grid, block, sh, st>>>(
+        (const float*)x, xs, w, W, vec, E, extra, top, ngroups, keep, scale, normalize, corr, dense,
+        idx, wts);
+    return (int)hipGetLastError();
+}
+
+int nx_latent_row(const void* x, long xs, int is_bf16, const float* w, float eps,
+                  const float* inv_freq, int half, const int* pos, const int* slots, void* cache,
+                  long nslots, void* row, long rs, long ntok, int C, int R, hipStream_t st) {
+    if (ntok <= 0) return 0;
+    if (C <= 0 || R < 0 || 2 * half > R || (half > 0 && !inv_freq)) return -1;
+    dim3 grid((unsigned)((ntok + 3) / 4)), block(4 * WAVE);
+    if (is_bf16) latent_row_kernel<bf16><<<grid, block, 0, st>>>(
+        (const bf16*)x, xs, w, eps, inv_freq, half, pos, slots, (bf16*)cache, nslots, (bf16*)row,
+        rs, ntok, C, R);
+    else latent_row_kernel<float><<<grid, block, 0, st>>>(
+        (const float*)x, xs, w, eps, inv_freq, half, pos, slots, (float*)cache, nslots,
+        (float*)row, rs, ntok, C, R);
     return (int)hipGetLastError();
 }
 

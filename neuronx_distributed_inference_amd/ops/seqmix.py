@@ -645,6 +645,68 @@ def group_limited_router(logits, num_experts: int, top_k: int, n_groups: int = 1
                                     correction)
 
 
+FUSED_ROUTER_MAX_TOKENS = 512
+
+
+def route_tokens(x, weight, num_experts: int, top_k: int, n_groups: int = 1,
+                 keep_groups: int = 1, scale: float = 1.0, normalize: bool = False,
+                 correction=None):
+    """Router product and selection: fp32 logits ``x.float() @ weight.T`` (x
+    (T, hidden) in any dtype, weight (E + extra, hidden) fp32), then
+    :func:`group_limited_router`. Steps of few tokens do both in one launch;
+    larger ones take the library product first."""
+    T = x.shape[0]
+    if x.is_cuda and 0 < T <= FUSED_ROUTER_MAX_TOKENS and x.stride(-1) == 1:
+        lib = _load()
+        E, C = num_experts, weight.shape[0]
+        assert weight.dtype == torch.float32 and weight.is_contiguous()
+        assert weight.shape[1] == x.shape[1] and E % max(n_groups, 1) == 0 and top_k <= E
+        dense = torch.empty(T, C, dtype=torch.float32, device=x.device)
+        idx = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
+        wts = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
+        _check(lib.nx_router_fused(
+            _p(x), ctypes.c_long(x.stride(0)), _is_bf16(x), _p(weight), weight.shape[1], E, C - E,
+            top_k, max(n_groups, 1), max(min(keep_groups, n_groups), 1), ctypes.c_float(scale),
+            int(normalize), _p(None if correction is None else _f32(correction)),
+            _p(dense), _p(idx), _p(wts), ctypes.c_long(T), _stream()), "route_tokens")
+        return dense, idx, wts
+    logits = torch.nn.functional.linear(x.float(), weight)
+    return group_limited_router(logits, num_experts, top_k, n_groups, keep_groups, scale,
+                                normalize, correction=correction)
+
+
+def latent_row_write(x, norm_weight, eps: float, inv_freq, step: StepLayout, k_cache,
+                     slot_mapping, kv_rank: int, row=None):
+    """Cache row of a latent layer in one pass: x (B,S,kv_rank + rot) (a column
+    slice is fine) -> [rms_norm(x[..., :kv_rank]) * w | interleaved-pair rotary
+    of the rest] scattered into the paged ``k_cache`` (blocks, block, 1,
+    kv_rank + rot) at ``slot_mapping``; ``row`` (B,S,kv_rank + rot, dense)
+    also receives it when given."""
+    B, S, CR = x.shape
+    C, R = kv_rank, CR - kv_rank
+    if x.is_cuda:
+        lib = _load()
+        assert k_cache.is_contiguous() and k_cache.shape[2] * k_cache.shape[3] == CR
+        assert k_cache.dtype == x.dtype and x.stride(2) == 1
+        assert row is None or (row.is_contiguous() and row.dtype == x.dtype and row.shape == x.shape)
+        _check(lib.nx_latent_row(
+            _p(x), ctypes.c_long(_token_stride(x)), _is_bf16(x), _p(_f32(norm_weight)),
+            ctypes.c_float(eps), _p(_f32(inv_freq)), inv_freq.numel(), _p(step.positions),
+            _p(step.i32(slot_mapping)), _p(k_cache),
+            ctypes.c_long(k_cache.shape[0] * k_cache.shape[1]), _p(row),
+            ctypes.c_long(0 if row is None else CR), ctypes.c_long(B * S), C, R, _stream()),
+            "latent_row_write")
+        return row
+    r = torch.empty(B, S, CR, dtype=x.dtype, device=x.device)
+    r[..., :C] = ref.rms_norm_rows(x[..., :C], norm_weight, eps, False, x.dtype)
+    r[..., C:] = ref.rotate_interleaved(x[..., C:].unsqueeze(2), step.positions,
+                                        inv_freq).squeeze(2).to(x.dtype)
+    ref.paged_kv_write(k_cache, None, r.view(B * S, 1, CR), None, slot_mapping)
+    if row is not None:
+        row.copy_(r)
+    return row
+
+
 def relu2_scale(hid, gates, expert_ff: int, num_experts: int, out_dtype=None):
     """relu(x)^2 of (T, E*ff + rest) pre-activations times the token's gate of
     the column's expert; the remaining columns take gate column E (see

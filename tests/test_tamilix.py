@@ -332,6 +332,83 @@ def test_plain_relu_squared_and_sigmoid_gate(device, C):
     close(got.cpu(), y.double() * torch.sigmoid(gate.double()), 1e-6)
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("T,W,E,extra", [(5, 24, 7, 0), (64, 64, 18, 0), (9, 136, 5, 2),
+                                         (600, 32, 9, 1)])
+def test_router_product_and_selection_in_one_call(device, T, W, E, extra):
+    """Few tokens: product and selection in one launch; many: the library
+    product first. Both equal the selection on float64 logits."""
+    torch.manual_seed(7)
+    wide = torch.randn(T, W + 8)
+    x = wide[:, 8:]                                      # a column slice, read in place
+    w = torch.randn(E + extra, W) * 0.5
+    corr = torch.randn(E) * 0.2
+    s = torch.softmax(x.double() @ w[:E].double().T, -1)
+    want_idx = torch.topk(s + corr.double(), 3 if E > 3 else 1, dim=-1).indices
+    top = want_idx.shape[1]
+    dense_w, idx, wts = seqmix.route_tokens(wide.to(device)[:, 8:], w.to(device), E, top,
+                                            correction=corr.to(device))
+    assert torch.equal(idx.long().cpu().sort(-1).values, want_idx.sort(-1).values)
+    close(wts.cpu(), torch.gather(s, 1, idx.long().cpu()), 2e-6)
+    assert dense_w.shape == (T, E + extra)
+    if extra:
+        close(dense_w[:, E:].cpu(), torch.sigmoid(x.double() @ w[E:].double().T), 2e-6)
+
+
+@pytest.mark.gpu
+def test_router_one_launch_bf16_input_gpu():
+    torch.manual_seed(8)
+    x = torch.randn(33, 256).bfloat16()
+    w = torch.randn(14, 256) * 0.2
+    s = torch.softmax(x.double() @ w.double().T, -1)
+    want_idx = torch.topk(s, 4, dim=-1).indices
+    _, idx, wts = seqmix.route_tokens(x.cuda(), w.cuda(), 14, 4)
+    assert torch.equal(idx.long().cpu().sort(-1).values, want_idx.sort(-1).values)
+    close(wts.cpu(), torch.gather(s, 1, idx.long().cpu()), 2e-6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("C,R,dims", [(10, 4, 4), (12, 8, 4), (64, 32, 32), (5, 2, 2)])
+def test_latent_cache_row_in_one_call(device, C, R, dims):
+    """Norm, rotation and the scatter into page slots; pad tokens and stale
+    pages stay as they are."""
+    from neuronx_distributed_inference_amd.modules.rope import interleaved_inv_freq
+
+    torch.manual_seed(9)
+    B, S, page, nblk = 2, 5, 4, 6
+    wide = torch.randn(B, S, C + R + 3) * 2
+    x = wide[..., 3:]
+    w = 1 + 0.3 * torch.randn(C)
+    pos = torch.tensor([[900, 901, 902, 903, 904], [0, 1, 2, -1, -1]])
+    slots = torch.tensor([[17, 18, 19, 4, 5], [9, 10, 11, -1, -1]])
+    cache = torch.randn(nblk, page, 1, C + R)
+    before = cache.clone()
+    st = seqmix.StepLayout(pos.to(device), torch.tensor([0, 1]).to(device))
+    inv = interleaved_inv_freq(100.0, dims)
+    cd = cache.clone().to(device)
+    row = torch.zeros(B, S, C + R, device=device)
+    seqmix.latent_row_write(wide.to(device)[..., 3:], w.to(device), EPS, inv.to(device), st, cd,
+                            slots.view(-1).to(device), C, row=row)
+    flat = cd.cpu().view(-1, C + R)
+    for b in range(B):
+        for t in range(S):
+            if pos[b, t] < 0:
+                continue
+            want = torch.cat([
+                oracle.norm(x[b, t, :C].double(), w.double(), EPS),
+                oracle.rotate_pairs(x[b, t, C:].double().view(1, 1, R), pos[b, t:t + 1], 100.0,
+                                    dims).view(R)])
+            close(flat[slots[b, t]], want, 3e-4)          # fp32 angles near position 900
+            close(row[b, t].cpu(), want, 3e-4)
+    untouched = torch.ones(nblk * page, dtype=torch.bool)
+    untouched[slots[slots >= 0]] = False
+    assert torch.equal(flat[untouched], before.view(-1, C + R)[untouched])
+    cd2 = cache.clone().to(device)                       # without the dense copy
+    seqmix.latent_row_write(wide.to(device)[..., 3:], w.to(device), EPS, inv.to(device), st, cd2,
+                            slots.view(-1).to(device), C)
+    assert torch.equal(cd2.cpu(), cd.cpu())
+
+
 def test_slope_ladder():
     for H in (1, 3, 8, 20):
         close(geometric_slopes(H), oracle.head_slopes(H), 1e-7)
